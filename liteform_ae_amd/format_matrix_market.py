@@ -1,0 +1,160 @@
+"""Matrix container for the CELL/hyb SpMM path.
+
+Mirrors the interface of the reference's ``format_matrix_market`` module
+(playground_pipline/format_matrix_market.py:12-205): ``Bucket`` is the cost-model
+record, ``MTX`` wraps a ``scipy.sparse.coo_matrix`` and hands out CSR/CSC/COO views.
+Anything that accepted a reference ``MTX`` accepts this one (same attribute and
+method names, same return types).
+
+Differences, all additive:
+  * ``MTX.from_coo`` / ``MTX.from_csr`` build a matrix from arrays without a file and
+    may keep real values (the reference forces every stored value to 1.0,
+    format_matrix_market.py:54, 63-64);
+  * the graph-dataset names of the reference need the ``dgl``/``ogb`` packages and a
+    network connection; they raise ``RuntimeError`` here.
+"""
+from __future__ import annotations
+
+from os.path import basename, splitext
+
+import numpy as np
+from scipy import sparse as sp
+
+__all__ = ["MTX", "Bucket"]
+
+_GRAPH_DATASETS = ("cora", "citeseer", "pubmed", "ppi", "arxiv", "proteins", "reddit")
+
+
+class Bucket:
+    """One (partition, width) bucket as the cost model sees it
+    (format_matrix_market.py:12-37)."""
+
+    def __init__(self, bucket_width: int, num_rows: int, nnz: int,
+                 row_indices: list, col_indices: set):
+        self.bucket_width = bucket_width
+        self.num_rows = num_rows
+        self.nnz = nnz
+        self.row_indices = row_indices
+        self.col_indices = col_indices
+
+    def __str__(self):
+        head = (f"Bucket(bucket_width={self.bucket_width}, num_rows={self.num_rows}, "
+                f"nnz={self.nnz}, len(row_indices)={len(self.row_indices)}, ")
+        if len(self.row_indices) < 11 and len(self.col_indices) < 11:
+            return (head + f"row_indices={self.row_indices}, "
+                    f"len(col_indices)={len(self.col_indices)}, col_indices={self.col_indices})")
+        return head + f"len(col_indices)={len(self.col_indices)})"
+
+
+class MTX:
+    """Sparse matrix held as scipy COO (format_matrix_market.py:40-205).
+
+    ``MTX(None)`` gives an empty shell whose ``coo_mtx`` the caller assigns;
+    ``MTX(path)`` reads a MatrixMarket file and sets every stored value to 1.
+    """
+
+    def __init__(self, filename):
+        self._csr = None
+        if filename is None:
+            self.name = None
+            self.coo_mtx = None
+        elif filename in _GRAPH_DATASETS:
+            raise RuntimeError(
+                f"dataset '{filename}' is downloaded through dgl/ogb in the reference; "
+                "those loaders are not part of this library - build the matrix with "
+                "MTX.from_coo / MTX.from_csr or pass a MatrixMarket path")
+        else:
+            from scipy.io import mmread
+            self.name = splitext(basename(filename))[0]
+            coo = sp.coo_matrix(mmread(filename))
+            coo.data = np.ones(len(coo.data))          # format_matrix_market.py:63-64
+            self.coo_mtx = coo
+
+    # ---- constructors without a file -------------------------------------------------
+    @classmethod
+    def from_coo(cls, row, col, shape, data=None, name=None):
+        m = cls(None)
+        m.name = name
+        row = np.asarray(row)
+        col = np.asarray(col)
+        if data is None:
+            data = np.ones(len(row))
+        m.coo_mtx = sp.coo_matrix((np.asarray(data), (row, col)), shape=shape)
+        return m
+
+    @classmethod
+    def from_csr(cls, indptr, indices, shape, data=None, name=None):
+        indptr = np.asarray(indptr)
+        indices = np.asarray(indices)
+        if data is None:
+            data = np.ones(len(indices))
+        csr = sp.csr_matrix((np.asarray(data), indices, indptr), shape=shape)
+        m = cls(None)
+        m.name = name
+        m.coo_mtx = csr.tocoo()
+        return m
+
+    def __setattr__(self, key, value):
+        if key == "coo_mtx":
+            object.__setattr__(self, "_csr", None)   # cached CSR follows the COO
+        object.__setattr__(self, key, value)
+
+    # ---- the reference's accessors ----------------------------------------------------
+    def _csr_view(self):
+        if self._csr is None:
+            object.__setattr__(self, "_csr", self.coo_mtx.tocsr())
+        return self._csr
+
+    def adj_tensors(self, format: str):
+        if format == "coo":
+            return self.coo_mtx.row, self.coo_mtx.col
+        elif format == "csc":
+            csc = self.coo_mtx.tocsc()
+            return csc.indptr, csc.indices, csc.data
+        elif format == "csr":
+            csr = self._csr_view()
+            return csr.indptr, csr.indices, csr.data
+        raise TypeError(f"Format {format} is not suppoted.")
+
+    def num_src_nodes(self):
+        return self.coo_mtx.shape[0]
+
+    def num_dst_nodes(self):
+        return self.coo_mtx.shape[1]
+
+    def num_edges(self):
+        return self.coo_mtx.nnz
+
+    def dot(self, B):
+        """A @ B through scipy (format_matrix_market.py:89-99)."""
+        return self.coo_mtx.tocsc().dot(B)
+
+    def tocsr(self, copy=False):
+        return self.coo_mtx.tocsr(copy=copy)
+
+    def matrix_features(self):
+        """Row-length statistics used by the format selector
+        (format_matrix_market.py:153-202)."""
+        num_rows, num_cols = self.coo_mtx.shape
+        indptr = self._csr_view().indptr
+        per_row = np.diff(indptr)
+        avg = np.mean(per_row)
+        lo = per_row.min()
+        hi = per_row.max()
+        return {
+            "name": self.name,
+            "num_rows": num_rows,
+            "num_cols": num_cols,
+            "nnz": self.coo_mtx.nnz,
+            "avg_nnz_per_row": avg,
+            "min_nnz_per_row": lo,
+            "max_nnz_per_row": hi,
+            "std_dev_nnz_per_row": np.std(per_row),
+            "avg_nnz_density_per_row": avg / num_cols,
+            "min_nnz_density_per_row": lo / num_cols,
+            "max_nnz_density_per_row": hi / num_cols,
+            "std_dev_nnz_density_per_row": np.std(per_row / num_cols),
+        }
+
+    def __str__(self):
+        return str(self.coo_mtx)

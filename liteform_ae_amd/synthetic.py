@@ -1,0 +1,178 @@
+"""Seeded synthetic matrices for the five benchmark workloads.
+
+Every generator returns a canonical CSR matrix (sorted columns, no duplicates,
+int32 indices) wrapped in :class:`MTX`, with real float32 values, plus the dense
+operand's shape and dtype.  ``scale`` shrinks the row/column counts so the same
+distribution can be used at test sizes; ``scale=1`` is the full workload.
+Seeds are 1000 + workload number.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+from scipy import sparse as sp
+
+from .format_matrix_market import MTX
+
+__all__ = ["Workload", "make_workload", "make_dense", "WORKLOADS", "csr_from_row_degrees"]
+
+
+@dataclass
+class Workload:
+    name: str
+    matrix: MTX
+    feat_size: int          # N, columns of the dense operand
+    num_parts: int          # column partitions (0 = let the chooser decide)
+    b_dtype: str            # "f32" or "bf16"
+    seed: int
+    description: str
+
+    @property
+    def shape(self):
+        return self.matrix.coo_mtx.shape
+
+    @property
+    def nnz(self):
+        return self.matrix.num_edges()
+
+
+def _mtx_from_csr(indptr, indices, data, shape, name):
+    csr = sp.csr_matrix((data, indices, indptr), shape=shape)
+    m = MTX(None)
+    m.name = name
+    m.coo_mtx = csr.tocoo()
+    object.__setattr__(m, "_csr", csr)
+    return m
+
+
+def csr_from_row_degrees(deg, num_cols, rng):
+    """Uniform neighbours for the given row degrees; duplicates inside a row are
+    dropped, so a row can end up slightly shorter than asked."""
+    deg = np.asarray(deg, dtype=np.int64)
+    num_rows = len(deg)
+    total = int(deg.sum())
+    key = np.repeat(np.arange(num_rows, dtype=np.int64), deg)
+    key *= num_cols
+    key += rng.integers(0, num_cols, size=total, dtype=np.int64)
+    key.sort()
+    keep = np.empty(total, dtype=bool)
+    keep[:1] = True
+    np.not_equal(key[1:], key[:-1], out=keep[1:])
+    key = key[keep]
+    row = key // num_cols
+    col = (key - row * num_cols).astype(np.int32)
+    counts = np.bincount(row, minlength=num_rows)
+    indptr = np.zeros(num_rows + 1, dtype=np.int64)
+    np.cumsum(counts, out=indptr[1:])
+    idt = np.int32 if indptr[-1] < 2**31 else np.int64
+    return indptr.astype(idt), col
+
+
+def _cfg1(scale, rng):
+    n = max(8, int(round(4096 * scale)))
+    deg = np.minimum(rng.poisson(16, size=n), n)
+    indptr = np.zeros(n + 1, dtype=np.int32)
+    indptr[1:] = np.cumsum(deg)
+    indices = np.empty(indptr[-1], dtype=np.int32)
+    for r in range(n):                                   # without replacement per row
+        indices[indptr[r]:indptr[r + 1]] = np.sort(rng.choice(n, size=deg[r], replace=False))
+    data = rng.uniform(-1.0, 1.0, size=indptr[-1]).astype(np.float32)
+    return indptr, indices, data, (n, n)
+
+
+def _cfg2(scale, rng):
+    n = max(64, int(round(170_000 * scale)))
+    deg = np.clip(rng.zipf(2.1, size=n), 1, min(13_000, n))
+    indptr, indices = csr_from_row_degrees(deg, n, rng)
+    rowlen = np.diff(indptr)
+    data = np.repeat((1.0 / np.maximum(rowlen, 1)).astype(np.float32), rowlen)
+    return indptr, indices, data, (n, n)
+
+
+def _cfg3(scale, rng):
+    n = max(64, int(round(2_450_000 * scale)))
+    deg = np.clip(np.rint(rng.lognormal(2.9, 1.1, size=n)), 1, min(17_000, n)).astype(np.int64)
+    indptr, indices = csr_from_row_degrees(deg, n, rng)
+    data = rng.random(size=indptr[-1], dtype=np.float32)
+    return indptr, indices, data, (n, n)
+
+
+def _cfg4(scale, rng):
+    g = max(3, int(round(100 * scale ** (1.0 / 3.0))))
+    n = g ** 3
+    idx = np.arange(n, dtype=np.int64)
+    x, y, z = idx % g, (idx // g) % g, idx // (g * g)
+    rows, cols = [], []
+    for dz in (-1, 0, 1):
+        for dy in (-1, 0, 1):
+            for dx in (-1, 0, 1):
+                ok = ((x + dx >= 0) & (x + dx < g) & (y + dy >= 0) & (y + dy < g)
+                      & (z + dz >= 0) & (z + dz < g))
+                rows.append(idx[ok])
+                cols.append(idx[ok] + dx + dy * g + dz * g * g)
+    rows = np.concatenate(rows)
+    cols = np.concatenate(cols)
+    csr = sp.csr_matrix((np.ones(len(rows), dtype=np.float32), (rows, cols)), shape=(n, n))
+    csr.sort_indices()
+    data = rng.standard_normal(size=csr.nnz).astype(np.float32)
+    return csr.indptr.astype(np.int32), csr.indices.astype(np.int32), data, (n, n)
+
+
+def _cfg5(scale, rng):
+    nr = max(64, int(round(500_000 * scale)))
+    nc = max(256, int(round(2_000_000 * scale)))
+    deg = np.floor(2.0 * (1.0 + rng.pareto(1.5, size=nr))).astype(np.int64)
+    deg = np.clip(deg, 2, nc)
+    n_dense = max(1, int(round(50 * min(1.0, scale * 4)))) if scale < 1 else 50
+    dense_len = min(nc, max(2048, int(round(100_000 * scale)))) if scale < 1 else 100_000
+    dense_rows = rng.choice(nr, size=n_dense, replace=False)
+    deg[dense_rows] = 0
+    indptr, indices = csr_from_row_degrees(deg, nc, rng)
+    # splice the dense rows in (columns without replacement)
+    rowlen = np.diff(indptr).astype(np.int64)
+    rowlen[dense_rows] = dense_len
+    new_ptr = np.zeros(nr + 1, dtype=np.int64)
+    np.cumsum(rowlen, out=new_ptr[1:])
+    new_idx = np.empty(new_ptr[-1], dtype=np.int32)
+    is_dense = np.zeros(nr, dtype=bool)
+    is_dense[dense_rows] = True
+    sparse_rows = np.nonzero(~is_dense)[0]
+    dst = np.repeat(new_ptr[sparse_rows] - indptr[sparse_rows], np.diff(indptr)[sparse_rows]) \
+        + np.arange(indptr[-1], dtype=np.int64)
+    new_idx[dst] = indices
+    for r in dense_rows:
+        new_idx[new_ptr[r]:new_ptr[r + 1]] = np.sort(
+            rng.choice(nc, size=dense_len, replace=False)).astype(np.int32)
+    data = rng.uniform(-1.0, 1.0, size=new_ptr[-1]).astype(np.float32)
+    idt = np.int32 if new_ptr[-1] < 2**31 else np.int64
+    return new_ptr.astype(idt), new_idx, data, (nr, nc)
+
+
+WORKLOADS = {
+    #  name: (generator, N, num_parts, B dtype, description)
+    "cfg1": (_cfg1, 32, 1, "f32", "uniform random 4096x4096, row nnz ~ Poisson(16), values U(-1,1)"),
+    "cfg2": (_cfg2, 128, 2, "f32", "power-law 170k x 170k, out-degree ~ Zipf(2.1) in [1,13000], values 1/deg"),
+    "cfg3": (_cfg3, 128, 0, "f32", "power-law 2.45M x 2.45M, degree ~ lognormal(2.9,1.1) in [1,17000], values U(0,1)"),
+    "cfg4": (_cfg4, 256, 1, "f32", "27-point stencil on a 100^3 grid, values N(0,1)"),
+    "cfg5": (_cfg5, 512, 0, "bf16", "skewed 500k x 2M, row nnz ~ Pareto(1.5, 2) plus 50 rows of 100k, values U(-1,1)"),
+}
+
+
+def make_workload(name: str, scale: float = 1.0, feat_size: int | None = None) -> Workload:
+    gen, n_feat, parts, b_dtype, desc = WORKLOADS[name]
+    seed = 1000 + int(name[3:])
+    rng = np.random.default_rng(seed)
+    indptr, indices, data, shape = gen(scale, rng)
+    mtx = _mtx_from_csr(indptr, indices, data, shape, name if scale == 1.0 else f"{name}@{scale:g}")
+    return Workload(name=name, matrix=mtx, feat_size=feat_size or n_feat, num_parts=parts,
+                    b_dtype=b_dtype, seed=seed, description=desc)
+
+
+def make_dense(num_rows: int, feat_size: int, seed: int) -> np.ndarray:
+    """Dense operand B: U(-1,1) float32, row-major (num_rows, feat_size)."""
+    rng = np.random.default_rng(seed + 7919)
+    b = rng.random(size=(num_rows, feat_size), dtype=np.float32)
+    b *= 2.0
+    b -= 1.0
+    return b
