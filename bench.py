@@ -1,0 +1,237 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused hyb SpMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3] [--feat 128] [--parts 1]
+
+A step is one SpMM  C = A_hyb . B  over the whole synthetic matrix, with A's hyb slabs, B and
+C resident in HBM.  The default workload is the 2.45M-row power-law graph at N = 128, the
+configuration the headline metric is quoted on.  Prints one JSON line:
+
+  value            GFLOP/s = 2 * nnz * N / t, from the wall time of K back-to-back steps
+  roofline         HBM: algorithmic bytes per step / average kernel time of a step measured
+                   with HIP events on the launch stream; traffic = L2<->fabric bytes per
+                   step from rocprofv3 counters when a measurement is on file
+  format_compose   bucket-width search and slab build times (GPU), reported beside it
+  cpu_baseline     scipy CSR @ dense (the reference's own CPU product, one thread) on a
+                   bounded sample of rows of the same matrix
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes(nnz, rows, cols, feat, b_bytes):
+    """A as CSR once, B once, C once."""
+    return nnz * 8 + (rows + 1) * 4 + cols * feat * b_bytes + rows * feat * 4
+
+
+def gather_bytes(nnz, rows, feat, b_bytes):
+    """The same with one B row fetched per nonzero (no reuse of B)."""
+    return nnz * 8 + (rows + 1) * 4 + nnz * feat * b_bytes + rows * feat * 4
+
+
+def recorded_traffic(workload, feat, parts):
+    """L2<->fabric bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(path):
+        return None
+    try:
+        table = json.load(open(path))
+    except Exception:
+        return None
+    return table.get(f"{workload}/N{feat}/P{parts}")
+
+
+def cpu_baseline(wl, B_host, feat, budget_s=20.0):
+    """scipy CSR(f32) @ dense(f32) on the first rows of the matrix, sized to ~budget_s."""
+    import scipy.sparse as sp
+    indptr, indices, data = wl.matrix.adj_tensors("csr")
+    rows = wl.shape[0]
+    nnz = int(indptr[-1])
+    # ~1 GFLOP/s is typical for scipy's single-threaded csr_matvecs at this width
+    target_nnz = int(budget_s * 1.0e9 / (2 * feat))
+    if nnz <= target_nnz:
+        take = rows
+    else:
+        take = int(np.searchsorted(indptr, target_nnz))
+        take = max(1, min(rows, take))
+    sub_nnz = int(indptr[take])
+    A = sp.csr_matrix((np.asarray(data[:sub_nnz], dtype=np.float32), indices[:sub_nnz], indptr[:take + 1]),
+                      shape=(take, wl.shape[1]))
+    Bf = np.ascontiguousarray(B_host, dtype=np.float32)
+    t0 = time.perf_counter()
+    out = A @ Bf
+    dt = time.perf_counter() - t0
+    return {
+        "value": round(2.0 * sub_nnz * feat / dt / 1e9, 3),
+        "unit": "GFLOP/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"scipy csr_matrix(f32) @ dense(f32), first {take} of {rows} rows "
+                  f"({sub_nnz} nnz), 1 run, {dt:.2f} s",
+    }, out, take
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg3")
+    ap.add_argument("--feat", type=int, default=0, help="dense columns N (default: the workload's)")
+    ap.add_argument("--parts", type=int, default=0, help="column partitions (default: the workload's, or 1)")
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink the matrix (testing only)")
+    ap.add_argument("--cost-model", default="reference", choices=["reference", "gfx950"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from liteform_ae_amd import _lib
+    from liteform_ae_amd import format_algos as fa
+    from liteform_ae_amd.synthetic import make_dense, make_workload
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    _lib.load()
+    torch.cuda.set_device(0)
+
+    t0 = time.perf_counter()
+    wl = make_workload(args.workload, args.scale)
+    feat = args.feat or wl.feat_size
+    parts = args.parts or wl.num_parts or 1
+    g = wl.matrix
+    rows, cols = wl.shape
+    nnz = wl.nnz
+    t_gen = time.perf_counter() - t0
+    print(f"[bench] {wl.name}: {rows} x {cols}, nnz {nnz}, N {feat}, P {parts}, B {wl.b_dtype} "
+          f"(generated in {t_gen:.1f} s)", file=sys.stderr, flush=True)
+
+    B_host = make_dense(cols, feat, wl.seed)
+    if wl.b_dtype == "bf16":
+        B_dev = torch.from_numpy(B_host).cuda().to(torch.bfloat16)
+        B_host = B_dev.to(torch.float32).cpu().numpy()      # what the kernel really reads
+        b_bytes = 2
+    else:
+        B_dev = torch.from_numpy(B_host).cuda()
+        b_bytes = 4
+    C_dev = torch.empty((rows, feat), dtype=torch.float32, device="cuda")
+
+    # ---- format composition (GPU): search = what the reference times as time_bucket
+    fa._device_csr(g)                       # upload CSR once, outside the timed parts
+    torch.cuda.synchronize()
+    cfg_obj = fa.CostModelSettings(feat, parts, cost_model=args.cost_model)
+    fa.search_bucket_config(g, parts, cfg_obj)            # warm
+    t0 = time.perf_counter()
+    config = fa.search_bucket_config(g, parts, cfg_obj)
+    search_ms = (time.perf_counter() - t0) * 1e3
+    fa.build_hyb_format_device(g, config)                 # warm
+    t0 = time.perf_counter()
+    fmt = fa.build_hyb_format_device(g, config)
+    build_ms = (time.perf_counter() - t0) * 1e3
+    plan = fa.HybSpMM(fmt, feat, wl.b_dtype)
+    print(f"[bench] config {config}; search {search_ms:.2f} ms, build {build_ms:.2f} ms; plan {plan.info}",
+          file=sys.stderr, flush=True)
+
+    # ---- timed region: K steps, inputs resident, synchronize on both sides
+    for _ in range(args.warmup):
+        plan.run(B_dev, C_dev)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.run(B_dev, C_dev)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+
+    # per-step kernel time from HIP events on the launch stream (warm caches, then flushed)
+    ev_ms = plan.time_ms(B_dev, C_dev, warmup=0, repeat=args.steps)
+    flush = torch.empty(int(512e6), dtype=torch.int8, device="cuda")
+    ev_cold_ms = plan.time_ms(B_dev, C_dev, warmup=0, repeat=max(3, args.steps // 3), flush=flush)
+    del flush
+    kernel_ms = float(np.mean(ev_ms))
+
+    flops = 2.0 * nnz * feat
+    algo = algorithmic_bytes(nnz, rows, cols, feat, b_bytes)
+    gath = gather_bytes(nnz, rows, feat, b_bytes)
+    achieved = algo / (kernel_ms * 1e-3) / 1e9
+    traffic = recorded_traffic(wl.name if args.scale == 1.0 else "", feat, parts)
+
+    result = {
+        "metric": "SpMM GFLOP/s & % HBM roofline at N=128; format-compose ms",
+        "value": round(flops / (ms_per_step * 1e-3) / 1e9, 2),
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if wl.b_dtype == "f32" else "bf16 B, f32 accumulate",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{wl.name}: {wl.description}" + ("" if args.scale == 1.0 else f" (scale {args.scale})"),
+            "rows": rows, "cols": cols, "nnz": nnz, "feat_size": feat, "num_parts": parts,
+            "bucket_widths": config, "cost_model": args.cost_model,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 5),
+            "traffic": traffic,
+            "kernel_ms": round(kernel_ms, 4),
+            "kernel_ms_min": round(float(np.min(ev_ms)), 4),
+            "kernel_ms_cold": round(float(np.mean(ev_cold_ms)), 4),
+            "algorithmic_bytes": algo,
+            "gather_bytes": gath,
+            "gather_GBps": round(gath / (kernel_ms * 1e-3) / 1e9, 1),
+        },
+        "format_compose": {
+            "search_ms": round(search_ms, 3),
+            "build_ms": round(build_ms, 3),
+            "total_ms": round(search_ms + build_ms, 3),
+            "slab_slots": fmt.total_slots(),
+            "ell_rows": int(np.sum(fmt.ell_rows)),
+        },
+    }
+
+    if not args.no_cpu:
+        base, ref_rows, take = cpu_baseline(wl, B_host, feat, args.cpu_seconds)
+        base["host_cpus"] = os.cpu_count()
+        result["cpu_baseline"] = base
+        # the same rows from the GPU, against the 1e-5 * sum|a||b| bound
+        from oracle import liteform_oracle as O
+        indptr, indices, data = g.adj_tensors("csr")
+        sub = int(indptr[take])
+        bound = O.spmm_abs_bound(indptr[:take + 1], indices[:sub], data[:sub], (take, cols), B_host)
+        gpu_rows = C_dev[:take].cpu().numpy()
+        exact = O.spmm_csr_f64(indptr[:take + 1], indices[:sub], np.asarray(data[:sub], dtype=np.float32),
+                               (take, cols), B_host)
+        excess = float((np.abs(gpu_rows - exact) - 1e-5 * bound).max())
+        result["parity"] = {"rows_checked": take, "within_1e-5_bound": bool(excess <= 0),
+                            "max_abs_err": float(np.abs(gpu_rows - exact).max())}
+    plan.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

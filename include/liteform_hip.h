@@ -1,0 +1,203 @@
+/*
+ * liteform_hip.h - C ABI of liblfhip.so, the MI355X (gfx950) implementation of
+ * LiteForm's CELL/hyb SpMM path:
+ *
+ *     CSR -> bucket statistics -> bucket-width search -> hyb composition -> fused SpMM
+ *
+ * The reference (johnpzh/liteform_ae) is Python that reaches the GPU through TVM
+ * (playground_pipline/format_algos.py:543-578, 595, 601); it has no FFI of its own.
+ * Each entry point below names the reference function whose work it takes over.
+ *
+ * Conventions
+ *   - Every function returns an int status: LF_OK (0) or a negative LF_ERR_* code.
+ *     lf_last_error() returns a thread-local, human-readable message for the last
+ *     failure on the calling thread.  The library never aborts or exits.
+ *   - Pointers named d_* are device pointers (hipMalloc / torch-ROCm storage),
+ *     pointers named h_* are host pointers.  The caller allocates and owns all of
+ *     them; the library owns only what an lf_spmm_plan holds, released by
+ *     lf_spmm_destroy.
+ *   - lf_stream_t is a hipStream_t (NULL = the null stream).  Kernels are enqueued on
+ *     it; a function synchronises that stream only where it must return host data
+ *     (documented per function).
+ *   - Index arrays are int32, row-major; values are float32.  A matrix must have
+ *     fewer than 2^31 stored entries.
+ *   - Handles and workspaces must not be used from two threads at once.
+ */
+#ifndef LITEFORM_HIP_H
+#define LITEFORM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LF_VERSION 100 /* 0.1.0 */
+
+#define LF_OK 0
+#define LF_ERR_INVALID (-1)     /* bad argument (null pointer, size, non power-of-two width ...) */
+#define LF_ERR_TOO_SMALL (-2)   /* a column partition holds a single nonzero: the reference raises
+                                   ValueError("The partition is too small, only having 1 non-zero
+                                   element.") at format_algos.py:920-921 */
+#define LF_ERR_HIP (-3)         /* a HIP runtime call failed; message carries hipGetErrorString */
+#define LF_ERR_CONFIG (-4)      /* width list does not fit the matrix (a partition with nonzeros
+                                   has no widths: IndexError at format_algos.py:279) */
+#define LF_ERR_UNSUPPORTED (-5) /* outside the implemented range (feature size, nnz >= 2^31 ...) */
+#define LF_ERR_WORKSPACE (-6)   /* workspace smaller than lf_*_workspace_bytes() asked for */
+
+#define LF_MAX_CLASSES 11       /* initial widths 1,2,...,1024 (format_algos.py:821 width_limit) */
+#define LF_STATS_FIELDS 4       /* per class: cost-model rows, nnz, distinct rows, reserved */
+
+#define LF_DTYPE_F32 0
+#define LF_DTYPE_BF16 1
+
+#define LF_COST_REFERENCE 0     /* format_algos.py:1035-1166 bit for bit */
+#define LF_COST_GFX950 1        /* traffic model for MI355X; same search, different cost */
+
+typedef void* lf_stream_t;
+typedef struct lf_spmm_plan lf_spmm_plan;
+
+int lf_version(void);
+const char* lf_last_error(void);
+const char* lf_status_string(int status);
+
+/* ------------------------------------------------------------------------------------
+ * Bucket statistics.  Replaces get_init_buckets (format_algos.py:819-900): instead of
+ * materialising per-bucket row lists and column sets on the host it returns, per column
+ * partition p and initial width class k (width 2^k, capped at width_limit):
+ *     h_stats[p][k] = { cost-model rows, nnz, distinct rows, 0 }
+ * and a histogram over columns of "which classes touch this column":
+ *     h_colhist[p][m] = number of columns of partition p whose class bitmask is m
+ * from which the size of the column set of any union of classes follows.
+ *
+ * d_seg_deg (optional, [num_parts][num_rows] int32) carries per-(partition,row) degrees
+ * counted from raw COO triplets as the reference does (format_algos.py:846-849); when
+ * NULL the degrees are the CSR segment lengths (identical for duplicate-free input).
+ * Synchronises the stream before returning (host outputs).
+ * ------------------------------------------------------------------------------------ */
+size_t lf_stats_workspace_bytes(int64_t num_rows, int64_t num_cols, int32_t num_parts);
+
+int lf_bucket_stats(const int32_t* d_indptr, const int32_t* d_indices, const int32_t* d_seg_deg,
+                    int64_t num_rows, int64_t num_cols, int32_t num_parts, int32_t width_limit,
+                    void* d_workspace, size_t workspace_bytes,
+                    int64_t* h_stats,   /* [num_parts][LF_MAX_CLASSES][LF_STATS_FIELDS] */
+                    int64_t* h_colhist, /* [num_parts][1 << LF_MAX_CLASSES] */
+                    lf_stream_t stream);
+
+/* Per-(partition,row) degrees from COO triplets (format_algos.py:249-252, 846-849).
+ * d_seg_deg [num_parts][num_rows] is cleared and filled on the stream. */
+int lf_coo_degrees(const int32_t* d_coo_row, const int32_t* d_coo_col, int64_t nnz,
+                   int64_t num_rows, int64_t num_cols, int32_t num_parts,
+                   int32_t* d_seg_deg, lf_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * Bucket-width search on the host (no GPU work).  Replaces modify_single_row_buckets,
+ * get_bucket_config, modify_bucket_widths, move_largest_bucket, move_width_one_bucket and
+ * get_memory_cost (format_algos.py:623-648, 709-816, 903-954, 1035-1166), including dict
+ * insertion order, the stale key snapshot and the strict-< rule, in IEEE double without
+ * contraction.  cfg_feat_size / cfg_num_parts are CostModelSettings' two fields
+ * (format_algos.py:45-49).
+ *   h_widths  [num_parts][LF_MAX_CLASSES]  ascending widths per partition
+ *   h_nwidths [num_parts]                  how many are valid (0 for an empty partition)
+ *   h_trace_cost / h_trace_len (optional)  cost of every state the search visited, in
+ *                                          visiting order ([num_parts][LF_MAX_CLASSES+1])
+ * Returns LF_ERR_TOO_SMALL where the reference raises ValueError.
+ * ------------------------------------------------------------------------------------ */
+int lf_search_bucket_config(const int64_t* h_stats, const int64_t* h_colhist, int32_t num_parts,
+                            int32_t width_limit, int32_t cfg_feat_size, int32_t cfg_num_parts,
+                            int32_t cost_model, int32_t* h_widths, int32_t* h_nwidths,
+                            double* h_trace_cost, int32_t* h_trace_len);
+
+/* ------------------------------------------------------------------------------------
+ * hyb composition.  Replaces build_hyb_format (format_algos.py:226-385).
+ * Bucket k = (partition p, width index b) in row-major (p, b) order; widths of partition
+ * p are h_widths_flat[h_widths_off[p] .. h_widths_off[p+1]), ascending powers of two.
+ *
+ * lf_hyb_plan counts the ELL rows of every bucket (h_ell_rows[k]) and leaves per-block
+ * offsets in the workspace; it synchronises the stream.  lf_hyb_layout (host only) turns
+ * those counts into the flat layout: bucket k owns ELL rows [h_row_off[k], +R_k) of
+ * d_rows / d_meta and slots [h_slot_off[k], +R_k*W_k) of d_cols / d_vals / d_mask; offsets
+ * are padded so that every slab is 256-byte aligned, and h_total_rows / h_total_slots are
+ * the element counts to allocate.  The caller then calls lf_hyb_build with the same
+ * arguments and workspace.  Bucket contents are exactly the reference's: rows[e] = source
+ * row, cols / mask row-major (R, W) padded with (0, 0); vals carries A's values (d_values
+ * NULL = all ones, which makes vals == mask).  Padding between slabs is left unwritten.
+ *
+ * d_meta[e] describes ELL row e for the SpMM kernels: bits 0..10 = valid slots (1..W);
+ * bits 11..30 = number of consecutive ELL rows holding the same source row when e is the
+ * first of them, or e's index among them on a continuation row; bit 31 set on a
+ * continuation row.  It is an acceleration structure, not part of the reference format.
+ * ------------------------------------------------------------------------------------ */
+size_t lf_hyb_workspace_bytes(int64_t num_rows, int32_t num_parts, int32_t total_buckets);
+
+int lf_hyb_plan(const int32_t* d_indptr, const int32_t* d_indices, const int32_t* d_seg_deg,
+                int64_t num_rows, int64_t num_cols, int32_t num_parts,
+                const int32_t* h_widths_flat, const int32_t* h_widths_off,
+                void* d_workspace, size_t workspace_bytes,
+                int64_t* h_ell_rows, lf_stream_t stream);
+
+int lf_hyb_layout(const int64_t* h_ell_rows, const int32_t* h_widths_flat, int32_t total_buckets,
+                  int64_t* h_row_off, int64_t* h_slot_off, int64_t* h_total_rows, int64_t* h_total_slots);
+
+int lf_hyb_build(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values,
+                 const int32_t* d_seg_deg,
+                 int64_t num_rows, int64_t num_cols, int32_t num_parts,
+                 const int32_t* h_widths_flat, const int32_t* h_widths_off,
+                 const int64_t* h_ell_rows,
+                 void* d_workspace, size_t workspace_bytes,
+                 int32_t* d_rows, int32_t* d_meta, int32_t* d_cols, float* d_vals, float* d_mask,
+                 lf_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * Fused SpMM  C[num_rows][feat] = A_hyb . B[num_cols][feat].  Replaces the kernel that
+ * bench_hyb_with_config builds and launches (format_algos.py:388-605): one launch per
+ * column partition walks every bucket of that partition; partitions run in ascending
+ * order on the stream, partition 0 stores and later partitions add, so the result does
+ * not depend on scheduling and no atomics are used.  C needs no clearing.
+ *
+ * A bucket is described the way the reference passes it to the kernel
+ * (format_algos.py:552-578: values float32, rows int32, cols int32 row-major), plus the
+ * optional meta array of lf_hyb_build (NULL: derived from rows/vals at create time).
+ * The slabs must stay alive and unchanged while the plan exists.
+ * feat_size must be a multiple of 32 (float32 B) or 64 (bf16 B), at most 1024.
+ * ------------------------------------------------------------------------------------ */
+typedef struct lf_bucket_desc {
+    int32_t width;          /* W, power of two, 1..1024 */
+    int32_t part;           /* column partition this bucket belongs to */
+    int64_t num_ell_rows;   /* R */
+    const int32_t* d_rows;  /* [R]     */
+    const int32_t* d_cols;  /* [R][W]  */
+    const float* d_vals;    /* [R][W]  */
+    const int32_t* d_meta;  /* [R] or NULL */
+} lf_bucket_desc;
+
+int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int32_t num_buckets,
+                   int32_t num_parts, int64_t num_rows, int64_t num_cols, int32_t feat_size,
+                   int32_t b_dtype, lf_stream_t stream);
+int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t stream);
+int lf_spmm_destroy(lf_spmm_plan* plan);
+
+/* h_info[0..7] = tiles, workgroups per launch, launches per run, LDS bytes per workgroup,
+ * heavy (split) segments, partial rows, rows cleared by partition 0, reserved. */
+int lf_spmm_info(const lf_spmm_plan* plan, int64_t* h_info);
+
+/* Timing helper, the counterpart of the reference's profile_tvm_ms / run_100_times
+ * (format_algos.py:164-202, 601): `warmup` untimed runs, then `repeat` runs each bracketed
+ * by HIP events on `stream`; before every timed run d_flush (if not NULL) is overwritten
+ * to evict the caches, as the reference zeroes a 256 MB buffer.  h_ms receives `repeat`
+ * kernel durations in milliseconds (all launches of one run together). Synchronises. */
+int lf_spmm_time_ms(lf_spmm_plan* plan, const void* d_B, float* d_C, int32_t warmup,
+                    int32_t repeat, void* d_flush, size_t flush_bytes, float* h_ms,
+                    lf_stream_t stream);
+
+/* Row-parallel CSR SpMM, the counterpart of bench_naive's kernel
+ * (format_algos.py:1689-1755): C = A_csr . B with float32 values (NULL = ones). */
+int lf_csr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values,
+                int64_t num_rows, int64_t num_cols, int32_t feat_size, int32_t b_dtype,
+                const void* d_B, float* d_C, lf_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LITEFORM_HIP_H */

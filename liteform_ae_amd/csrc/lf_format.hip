@@ -1,0 +1,695 @@
+// Device side of format composition for gfx950: bucket statistics for the width search
+// and the hyb (column partition x power-of-two ELL bucket) builder.
+//
+// Reference behaviour reproduced here:
+//   get_init_buckets   playground_pipline/format_algos.py:819-900   (lf_bucket_stats)
+//   build_hyb_format   playground_pipline/format_algos.py:226-385   (lf_hyb_plan / lf_hyb_build)
+//
+// The reference walks nonzeros one at a time on the host.  On the GPU the same result is
+// obtained from per-(row, partition) segments: CSR is row-major with ascending columns,
+// so the nonzeros of one segment are contiguous, every bucket receives whole segments in
+// ascending row order, and a segment of `fill` entries occupies ceil(fill / W) consecutive
+// ELL rows that carry the same row id, with (0, 0) padding only after its last entry.
+// ELL-row offsets are therefore an exclusive scan, in row order, of per-segment ELL-row
+// counts, taken separately for each bucket.  All counting uses integer arithmetic, so the
+// output does not depend on scheduling.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+#include <vector>
+
+#include "lf_internal.h"
+
+namespace {
+
+constexpr int kBlock = 256;          // rows per workgroup in the per-segment kernels
+constexpr int kSlotsPerThread = 4;   // slab slots written per thread in the scatter
+constexpr int kLongSeg = 128;        // segments longer than this are walked by a whole wave
+// meta word of an ELL row: bits 0..10 valid slots (1..1024); bits 11..30 a count: on the
+// first ELL row of a source row's segment the number of ELL rows in the segment, on a
+// continuation row its index inside the segment; bit 31 set on continuation rows.
+constexpr int kMetaLenBits = 11;
+constexpr int kMetaSegMax = (1 << (31 - kMetaLenBits)) - 1;
+constexpr uint32_t kMetaCont = 0x80000000u;
+
+__host__ __device__ inline int32_t make_meta(int len, int i, int n_ell) {
+    return (int32_t)((uint32_t)len | ((uint32_t)(i == 0 ? n_ell : i) << kMetaLenBits) | (i == 0 ? 0u : kMetaCont));
+}
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// ---------------------------------------------------------------------------- device utils
+__device__ __forceinline__ int lower_bound_i32(const int32_t* __restrict__ a, int lo, int hi, int64_t key) {
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if ((int64_t)a[mid] < key) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
+// Segment (row r, partition p): offset of its first entry in the CSR arrays and its length.
+// With one partition the segment is the row; otherwise boundaries were precomputed into
+// bnd[(P + 1)][rows] (partition-major so that neighbouring threads read neighbouring words).
+struct SegView {
+    const int32_t* indptr;
+    const int32_t* bnd;
+    int64_t rows;
+    int parts;
+};
+
+__device__ __forceinline__ void seg_range(const SegView& v, int64_t r, int p, int& start, int& fill) {
+    if (v.parts == 1) {
+        start = v.indptr[r];
+        fill = v.indptr[r + 1] - start;
+    } else {
+        start = v.bnd[(int64_t)p * v.rows + r];
+        fill = v.bnd[(int64_t)(p + 1) * v.rows + r] - start;
+    }
+}
+
+__global__ void fill_u32_kernel(uint32_t* __restrict__ p, int64_t n, uint32_t value) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * blockDim.x)
+        p[i] = value;
+}
+
+hipError_t fill_u32(void* p, int64_t n_words, uint32_t value, hipStream_t s) {
+    if (n_words <= 0) return hipSuccess;
+    const int grid = (int)std::min<int64_t>((n_words + 255) / 256, 4096);
+    fill_u32_kernel<<<grid, 256, 0, s>>>((uint32_t*)p, n_words, value);
+    return hipGetLastError();
+}
+
+// bnd[p][r] = first CSR position of row r whose column is >= p * psize   (p = 0..P)
+__global__ void seg_bounds_kernel(const int32_t* __restrict__ indptr, const int32_t* __restrict__ indices,
+                                  int64_t rows, int parts, int64_t psize, int32_t* __restrict__ bnd) {
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    const int lo = indptr[r], hi = indptr[r + 1];
+    bnd[r] = lo;
+    int cur = lo;
+    for (int p = 1; p < parts; ++p) {
+        cur = lower_bound_i32(indices, cur, hi, (int64_t)p * psize);
+        bnd[(int64_t)p * rows + r] = cur;
+    }
+    bnd[(int64_t)parts * rows + r] = hi;
+}
+
+// deg[p][r] += 1 for every COO triplet (format_algos.py:846-849 counts raw triplets)
+__global__ void coo_degree_kernel(const int32_t* __restrict__ row, const int32_t* __restrict__ col,
+                                  int64_t nnz, int64_t rows, int64_t psize, int32_t* __restrict__ deg) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nnz;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t p = col[i] / psize;
+        atomicAdd(&deg[p * rows + row[i]], 1);
+    }
+}
+
+// Initial width class of a segment of `deg` entries: width = min(next_pow2(deg), limit),
+// cost-model rows = max(1, next_pow2(deg) / limit)            (format_algos.py:875-882)
+__device__ __forceinline__ void width_class(int deg, int kmax, int& k, int& cost_rows) {
+    k = deg <= 1 ? 0 : 32 - __clz(deg - 1);
+    cost_rows = 1;
+    if (k > kmax) {
+        cost_rows = 1 << (k - kmax);
+        k = kmax;
+    }
+}
+
+// One thread per (row, partition) segment; blockIdx.y is the partition.
+//   stats[p][k] += {cost rows, nnz, 1}
+//   colmask[c]  |= 1 << k        for every column c of the segment
+// Long segments are walked by the whole wave so that a heavy row does not serialise.
+__global__ void __launch_bounds__(kBlock)
+bucket_stats_kernel(SegView v, const int32_t* __restrict__ indices, const int32_t* __restrict__ seg_deg,
+                    int kmax, uint32_t* __restrict__ colmask, unsigned long long* __restrict__ stats) {
+    __shared__ unsigned long long s_stats[LF_MAX_CLASSES * LF_STATS_FIELDS];
+    for (int i = threadIdx.x; i < LF_MAX_CLASSES * LF_STATS_FIELDS; i += kBlock) s_stats[i] = 0ull;
+    __syncthreads();
+
+    const int p = blockIdx.y;
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    int start = 0, fill = 0, deg = 0;
+    if (r < v.rows) {
+        seg_range(v, r, p, start, fill);
+        deg = seg_deg ? seg_deg[(int64_t)p * v.rows + r] : fill;
+    }
+    uint32_t bit = 0;
+    if (deg > 0) {
+        int k, cost_rows;
+        width_class(deg, kmax, k, cost_rows);
+        bit = 1u << k;
+        atomicAdd(&s_stats[k * LF_STATS_FIELDS + 0], (unsigned long long)cost_rows);
+        atomicAdd(&s_stats[k * LF_STATS_FIELDS + 1], (unsigned long long)deg);
+        atomicAdd(&s_stats[k * LF_STATS_FIELDS + 2], 1ull);
+    }
+    const bool is_long = bit != 0 && fill > kLongSeg;
+    if (bit != 0 && !is_long) {
+        for (int i = 0; i < fill; ++i) {
+            const int c = indices[start + i];
+            if ((colmask[c] & bit) == 0) atomicOr(&colmask[c], bit);
+        }
+    }
+    unsigned long long pending = __ballot(is_long);
+    const int lane = threadIdx.x & 63;
+    while (pending) {
+        const int src = __ffsll((long long)pending) - 1;
+        pending &= pending - 1;
+        const int s = __shfl(start, src);
+        const int f = __shfl(fill, src);
+        const uint32_t b = (uint32_t)__shfl((int)bit, src);
+        for (int i = lane; i < f; i += 64) {
+            const int c = indices[s + i];
+            if ((colmask[c] & b) == 0) atomicOr(&colmask[c], b);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < LF_MAX_CLASSES * LF_STATS_FIELDS; i += kBlock)
+        if (s_stats[i]) atomicAdd(&stats[(size_t)p * LF_MAX_CLASSES * LF_STATS_FIELDS + i], s_stats[i]);
+}
+
+// hist[p][mask] = number of columns of partition p with that class mask
+__global__ void __launch_bounds__(kBlock)
+colmask_hist_kernel(const uint32_t* __restrict__ colmask, int64_t cols, int64_t psize,
+                    unsigned long long* __restrict__ hist) {
+    constexpr int kBins = 1 << LF_MAX_CLASSES;
+    __shared__ uint32_t s_hist[kBins];
+    for (int i = threadIdx.x; i < kBins; i += kBlock) s_hist[i] = 0;
+    __syncthreads();
+    const int p = blockIdx.y;
+    const int64_t lo = (int64_t)p * psize;
+    const int64_t hi = lo + psize < cols ? lo + psize : cols;
+    for (int64_t c = lo + (int64_t)blockIdx.x * kBlock + threadIdx.x; c < hi;
+         c += (int64_t)gridDim.x * kBlock)
+        atomicAdd(&s_hist[colmask[c] & (kBins - 1)], 1u);
+    __syncthreads();
+    for (int i = threadIdx.x; i < kBins; i += kBlock)
+        if (s_hist[i]) atomicAdd(&hist[(size_t)p * kBins + i], (unsigned long long)s_hist[i]);
+}
+
+// ---------------------------------------------------------------------------- hyb plan/build
+// Width table on the device: wtab[p][0] = count, wtab[p][1 + b] = width, wtab[p][12] = index
+// of the partition's first bucket in the flat (p, b) bucket order.
+constexpr int kWtabStride = 16;
+
+// Bucket of a segment: first width >= deg, else the widest (format_algos.py:275-279).
+__device__ __forceinline__ int pick_bucket(const int32_t* __restrict__ w, int n, int deg) {
+    int b = 0;
+    while (b < n && w[1 + b] < deg) ++b;
+    return b == n ? n - 1 : b;
+}
+
+// Per workgroup of kBlock rows and per bucket: number of ELL rows the block contributes.
+// blockcnt[(bucket_base[p] + b) * nblk + blk]
+__global__ void __launch_bounds__(kBlock)
+hyb_count_kernel(SegView v, const int32_t* __restrict__ seg_deg, const int32_t* __restrict__ wtab,
+                 int nblk, int32_t* __restrict__ blockcnt, int32_t* __restrict__ flags) {
+    __shared__ int s_cnt[LF_MAX_CLASSES];
+    if (threadIdx.x < LF_MAX_CLASSES) s_cnt[threadIdx.x] = 0;
+    __syncthreads();
+    const int p = blockIdx.y;
+    const int32_t* w = wtab + p * kWtabStride;
+    const int n = w[0];
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (r < v.rows) {
+        int start, fill;
+        seg_range(v, r, p, start, fill);
+        if (fill > 0) {
+            if (n == 0) {
+                atomicOr(&flags[0], 1);       // nonzeros in a partition without widths
+            } else {
+                const int deg = seg_deg ? seg_deg[(int64_t)p * v.rows + r] : fill;
+                const int b = pick_bucket(w, n, deg);
+                const int width = w[1 + b];
+                const int n_ell = (fill + width - 1) / width;
+                if (n_ell > kMetaSegMax) atomicOr(&flags[0], 2);
+                atomicAdd(&s_cnt[b], n_ell);
+            }
+        }
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < n)
+        blockcnt[(int64_t)(w[12] + threadIdx.x) * nblk + blockIdx.x] = s_cnt[threadIdx.x];
+}
+
+// Exclusive scan over blocks, one workgroup per bucket; totals[k] = ELL rows of bucket k.
+__global__ void __launch_bounds__(1024)
+hyb_scan_kernel(int32_t* __restrict__ blockcnt, int nblk, long long* __restrict__ totals) {
+    __shared__ long long s_wave[16];
+    __shared__ long long s_carry;
+    int32_t* a = blockcnt + (int64_t)blockIdx.x * nblk;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0) s_carry = 0;
+    __syncthreads();
+    for (int base = 0; base < nblk; base += 1024) {
+        const int i = base + threadIdx.x;
+        const long long x = i < nblk ? a[i] : 0;
+        long long incl = x;
+        for (int d = 1; d < 64; d <<= 1) {
+            const long long y = __shfl_up(incl, d);
+            if (lane >= d) incl += y;
+        }
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        long long wave_off = 0;
+        for (int wv = 0; wv < wave; ++wv) wave_off += s_wave[wv];
+        const long long carry = s_carry;
+        if (i < nblk) a[i] = (int32_t)(carry + wave_off + incl - x);
+        __syncthreads();
+        if (threadIdx.x == 1023) s_carry = carry + wave_off + incl;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) totals[blockIdx.x] = s_carry;
+}
+
+// Writes, for every ELL row, its source row and meta word.  The in-block position comes
+// from one block-wide exclusive scan per bucket.
+__global__ void __launch_bounds__(kBlock)
+hyb_rows_kernel(SegView v, const int32_t* __restrict__ seg_deg, const int32_t* __restrict__ wtab,
+                int nblk, const int32_t* __restrict__ blockoff, const long long* __restrict__ row_off,
+                int32_t* __restrict__ out_rows, int32_t* __restrict__ out_meta) {
+    __shared__ int s_wave[kBlock / 64];
+    const int p = blockIdx.y;
+    const int32_t* w = wtab + p * kWtabStride;
+    const int n = w[0];
+    const int kbase = w[12];
+    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+    int start = 0, fill = 0, mine = -1, width = 1, n_ell = 0;
+    if (r < v.rows && n > 0) {
+        seg_range(v, r, p, start, fill);
+        if (fill > 0) {
+            const int deg = seg_deg ? seg_deg[(int64_t)p * v.rows + r] : fill;
+            mine = pick_bucket(w, n, deg);
+            width = w[1 + mine];
+            n_ell = (fill + width - 1) / width;
+        }
+    }
+    long long first = 0;      // flat ELL-row index of this segment's first ELL row
+    for (int b = 0; b < n; ++b) {
+        const int x = mine == b ? n_ell : 0;
+        int incl = x;
+        for (int d = 1; d < 64; d <<= 1) {
+            const int y = __shfl_up(incl, d);
+            if (lane >= d) incl += y;
+        }
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        int wave_off = 0;
+        for (int wv = 0; wv < wave; ++wv) wave_off += s_wave[wv];
+        if (mine == b)
+            first = row_off[kbase + b] + blockoff[(int64_t)(kbase + b) * nblk + blockIdx.x] + wave_off + incl - x;
+        __syncthreads();
+    }
+    const bool is_long = n_ell > 8;
+    if (n_ell > 0 && !is_long) {
+        for (int i = 0; i < n_ell; ++i) {
+            const int len = min(width, fill - i * width);
+            out_rows[first + i] = (int32_t)r;
+            out_meta[first + i] = make_meta(len, i, n_ell);
+        }
+    }
+    unsigned long long pending = __ballot(is_long);
+    while (pending) {
+        const int src = __ffsll((long long)pending) - 1;
+        pending &= pending - 1;
+        const long long f0 = __shfl(first, src);
+        const int fl = __shfl(fill, src);
+        const int wd = __shfl(width, src);
+        const int ne = __shfl(n_ell, src);
+        const int rr = (int)((int64_t)blockIdx.x * kBlock + (wave << 6) + src);
+        for (int i = lane; i < ne; i += 64) {
+            const int len = min(wd, fl - i * wd);
+            out_rows[f0 + i] = rr;
+            out_meta[f0 + i] = make_meta(len, i, ne);
+        }
+    }
+}
+
+// One thread per kSlotsPerThread consecutive slab slots.  A bucket's slot range starts at a
+// workgroup boundary (slot_off is aligned to the workgroup's span), so a workgroup serves a
+// single bucket, found by a short search over block_start.
+struct ScatterBucket {
+    long long slot_off;    // first slot of the bucket in the flat slab arrays
+    long long row_off;     // first ELL row of the bucket in the flat row arrays
+    long long n_slots;     // R * W
+    int log_w;
+    int block_start;       // first workgroup serving this bucket
+    int part;              // column partition of the bucket
+    int pad_;
+};
+
+__global__ void __launch_bounds__(kBlock)
+hyb_scatter_kernel(const ScatterBucket* __restrict__ buckets, int nb, SegView v,
+                   const int32_t* __restrict__ indices, const float* __restrict__ values,
+                   const int32_t* __restrict__ rows, const int32_t* __restrict__ meta,
+                   int32_t* __restrict__ out_cols, float* __restrict__ out_vals, float* __restrict__ out_mask) {
+    int lo = 0, hi = nb - 1;
+    while (lo < hi) {                      // last bucket whose block_start <= blockIdx.x
+        const int mid = (lo + hi + 1) >> 1;
+        if (buckets[mid].block_start <= (int)blockIdx.x) lo = mid; else hi = mid - 1;
+    }
+    const ScatterBucket bk = buckets[lo];
+    const long long t0 = ((long long)(blockIdx.x - bk.block_start) * kBlock + threadIdx.x) * kSlotsPerThread;
+    if (t0 >= bk.n_slots) return;
+    const int wmask = (1 << bk.log_w) - 1;
+    int32_t c[kSlotsPerThread];
+    float x[kSlotsPerThread], m[kSlotsPerThread];
+#pragma unroll
+    for (int u = 0; u < kSlotsPerThread; ++u) {
+        const long long t = t0 + u;
+        c[u] = 0; x[u] = 0.f; m[u] = 0.f;
+        if (t < bk.n_slots) {
+            const long long e = bk.row_off + (t >> bk.log_w);
+            const int s = (int)(t & wmask);
+            const uint32_t mw = (uint32_t)meta[e];
+            const int len = (int)(mw & ((1u << kMetaLenBits) - 1));
+            if (s < len) {
+                int start, fill;
+                seg_range(v, rows[e], bk.part, start, fill);
+                const int idx = (mw & kMetaCont) ? (int)((mw & ~kMetaCont) >> kMetaLenBits) : 0;
+                const int at = start + (idx << bk.log_w) + s;
+                c[u] = indices[at];
+                x[u] = values ? values[at] : 1.0f;
+                m[u] = 1.0f;
+            }
+        }
+    }
+    const long long o = bk.slot_off + t0;
+    if (t0 + kSlotsPerThread <= bk.n_slots) {      // slot_off and t0 are multiples of 4
+        *reinterpret_cast<int4*>(out_cols + o) = make_int4(c[0], c[1], c[2], c[3]);
+        *reinterpret_cast<float4*>(out_vals + o) = make_float4(x[0], x[1], x[2], x[3]);
+        if (out_mask) *reinterpret_cast<float4*>(out_mask + o) = make_float4(m[0], m[1], m[2], m[3]);
+    } else {
+        for (int u = 0; u < kSlotsPerThread && t0 + u < bk.n_slots; ++u) {
+            out_cols[o + u] = c[u];
+            out_vals[o + u] = x[u];
+            if (out_mask) out_mask[o + u] = m[u];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------- host helpers
+struct StatsLayout {
+    size_t bnd, colmask, stats, hist, total;
+};
+
+StatsLayout stats_layout(int64_t rows, int64_t cols, int parts) {
+    StatsLayout L{};
+    size_t off = 0;
+    L.bnd = off;
+    if (parts > 1) off += align_up((size_t)(parts + 1) * rows * 4, 256);
+    L.colmask = off;
+    off += align_up((size_t)cols * 4, 256);
+    L.stats = off;
+    off += align_up((size_t)parts * LF_MAX_CLASSES * LF_STATS_FIELDS * 8, 256);
+    L.hist = off;
+    off += align_up((size_t)parts * (1 << LF_MAX_CLASSES) * 8, 256);
+    L.total = off;
+    return L;
+}
+
+struct HybLayout {
+    size_t bnd, wtab, flags, totals, row_off, scatter, blockcnt, total;
+    int nblk;
+};
+
+HybLayout hyb_layout(int64_t rows, int parts, int total_buckets) {
+    HybLayout L{};
+    L.nblk = (int)((rows + kBlock - 1) / kBlock);
+    if (L.nblk < 1) L.nblk = 1;
+    size_t off = 0;
+    L.bnd = off;
+    if (parts > 1) off += align_up((size_t)(parts + 1) * rows * 4, 256);
+    L.wtab = off;
+    off += align_up((size_t)parts * kWtabStride * 4, 256);
+    L.flags = off;
+    off += 256;
+    L.totals = off;
+    off += align_up((size_t)std::max(total_buckets, 1) * 8, 256);
+    L.row_off = off;
+    off += align_up((size_t)std::max(total_buckets, 1) * 8, 256);
+    L.scatter = off;
+    off += align_up((size_t)std::max(total_buckets, 1) * sizeof(ScatterBucket), 256);
+    L.blockcnt = off;
+    off += align_up((size_t)std::max(total_buckets, 1) * L.nblk * 4, 256);
+    L.total = off;
+    return L;
+}
+
+// Flat slab layout shared by the builder and its callers: ELL rows of bucket k start at a
+// multiple of 64 entries, its slots at a multiple of the scatter workgroup span (1024
+// slots), so every slab is at least 256-byte aligned inside 256-byte aligned allocations.
+constexpr int64_t kRowAlign = 64;
+constexpr int64_t kSlotAlign = (int64_t)kBlock * kSlotsPerThread;
+
+void flat_layout(const int64_t* ell_rows, const int32_t* widths, int nb, int64_t* row_off,
+                 int64_t* slot_off, int64_t* total_rows, int64_t* total_slots) {
+    int64_t r = 0, s = 0;
+    for (int k = 0; k < nb; ++k) {
+        row_off[k] = r;
+        slot_off[k] = s;
+        r += (ell_rows[k] + kRowAlign - 1) / kRowAlign * kRowAlign;
+        s += (ell_rows[k] * widths[k] + kSlotAlign - 1) / kSlotAlign * kSlotAlign;
+    }
+    *total_rows = r;
+    *total_slots = s;
+}
+
+int check_common(const int32_t* d_indptr, const int32_t* d_indices, int64_t rows, int64_t cols, int parts) {
+    LF_REQUIRE(d_indptr != nullptr, LF_ERR_INVALID, "indptr is null");
+    LF_REQUIRE(rows >= 0 && cols >= 1, LF_ERR_INVALID, "bad shape %lld x %lld", (long long)rows, (long long)cols);
+    LF_REQUIRE(rows < (1ll << 31) && cols < (1ll << 31), LF_ERR_UNSUPPORTED, "shape exceeds int32 indices");
+    LF_REQUIRE(parts >= 1 && parts <= 65535, LF_ERR_INVALID, "num_parts must be in 1..65535 (got %d)", parts);
+    (void)d_indices;
+    return LF_OK;
+}
+
+int check_widths(int parts, const int32_t* flat, const int32_t* off) {
+    LF_REQUIRE(flat && off, LF_ERR_INVALID, "width table is null");
+    LF_REQUIRE(off[0] == 0, LF_ERR_INVALID, "widths_off[0] must be 0");
+    for (int p = 0; p < parts; ++p) {
+        const int n = off[p + 1] - off[p];
+        LF_REQUIRE(n >= 0 && n <= LF_MAX_CLASSES, LF_ERR_INVALID,
+                   "partition %d has %d widths (max %d)", p, n, LF_MAX_CLASSES);
+        for (int b = 0; b < n; ++b) {
+            const int w = flat[off[p] + b];
+            LF_REQUIRE(lf::is_pow2(w) && w <= (1 << (LF_MAX_CLASSES - 1)), LF_ERR_INVALID,
+                       "invalid padding for col_indices[%d][%d] and bucket_width=%d", p, b, w);
+            LF_REQUIRE(b == 0 || flat[off[p] + b - 1] < w, LF_ERR_INVALID,
+                       "widths of partition %d are not strictly ascending", p);
+        }
+    }
+    return LF_OK;
+}
+
+}  // namespace
+
+// ============================================================================ C ABI
+extern "C" {
+
+size_t lf_stats_workspace_bytes(int64_t num_rows, int64_t num_cols, int32_t num_parts) {
+    if (num_rows < 0 || num_cols < 0 || num_parts < 1) return 0;
+    return stats_layout(num_rows, num_cols, num_parts).total;
+}
+
+int lf_coo_degrees(const int32_t* d_coo_row, const int32_t* d_coo_col, int64_t nnz, int64_t num_rows,
+                   int64_t num_cols, int32_t num_parts, int32_t* d_seg_deg, lf_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    LF_REQUIRE(d_seg_deg, LF_ERR_INVALID, "seg_deg is null");
+    LF_REQUIRE(nnz == 0 || (d_coo_row && d_coo_col), LF_ERR_INVALID, "COO arrays are null");
+    LF_REQUIRE(num_parts >= 1 && num_cols >= 1, LF_ERR_INVALID, "bad num_parts / num_cols");
+    const int64_t psize = lf::ceil_div(num_cols, num_parts);
+    LF_HIP(fill_u32(d_seg_deg, (int64_t)num_parts * num_rows, 0u, s));
+    if (nnz > 0) {
+        const int grid = (int)std::min<int64_t>((nnz + 255) / 256, 65535);
+        coo_degree_kernel<<<grid, 256, 0, s>>>(d_coo_row, d_coo_col, nnz, num_rows, psize, d_seg_deg);
+        LF_HIP(hipGetLastError());
+    }
+    return LF_OK;
+}
+
+int lf_bucket_stats(const int32_t* d_indptr, const int32_t* d_indices, const int32_t* d_seg_deg,
+                    int64_t num_rows, int64_t num_cols, int32_t num_parts, int32_t width_limit,
+                    void* d_workspace, size_t workspace_bytes, int64_t* h_stats, int64_t* h_colhist,
+                    lf_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (int rc = check_common(d_indptr, d_indices, num_rows, num_cols, num_parts)) return rc;
+    LF_REQUIRE(h_stats && h_colhist, LF_ERR_INVALID, "output pointers are null");
+    LF_REQUIRE(lf::is_pow2(width_limit) && width_limit <= (1 << (LF_MAX_CLASSES - 1)), LF_ERR_INVALID,
+               "width_limit must be a power of two <= %d", 1 << (LF_MAX_CLASSES - 1));
+    const StatsLayout L = stats_layout(num_rows, num_cols, num_parts);
+    LF_REQUIRE(d_workspace && workspace_bytes >= L.total, LF_ERR_WORKSPACE,
+               "workspace has %zu bytes, %zu needed", workspace_bytes, L.total);
+    char* ws = (char*)d_workspace;
+    int32_t* bnd = (int32_t*)(ws + L.bnd);
+    uint32_t* colmask = (uint32_t*)(ws + L.colmask);
+    unsigned long long* stats = (unsigned long long*)(ws + L.stats);
+    unsigned long long* hist = (unsigned long long*)(ws + L.hist);
+    const int64_t psize = lf::ceil_div(num_cols, num_parts);
+    const size_t stats_bytes = (size_t)num_parts * LF_MAX_CLASSES * LF_STATS_FIELDS * 8;
+    const size_t hist_bytes = (size_t)num_parts * (1 << LF_MAX_CLASSES) * 8;
+
+    LF_HIP(fill_u32(colmask, (L.total - L.colmask) / 4, 0u, s));   // colmask, stats and hist
+    if (num_rows > 0) {
+        const int nblk = (int)((num_rows + kBlock - 1) / kBlock);
+        if (num_parts > 1) {
+            seg_bounds_kernel<<<nblk, kBlock, 0, s>>>(d_indptr, d_indices, num_rows, num_parts, psize, bnd);
+            LF_HIP(hipGetLastError());
+        }
+        SegView v{d_indptr, bnd, num_rows, num_parts};
+        bucket_stats_kernel<<<dim3(nblk, num_parts), kBlock, 0, s>>>(v, d_indices, d_seg_deg,
+                                                                     lf::ilog2(width_limit), colmask, stats);
+        LF_HIP(hipGetLastError());
+        const int hgrid = (int)std::min<int64_t>((psize + kBlock - 1) / kBlock, 1024);
+        colmask_hist_kernel<<<dim3(hgrid, num_parts), kBlock, 0, s>>>(colmask, num_cols, psize, hist);
+        LF_HIP(hipGetLastError());
+    }
+    LF_HIP(hipMemcpyAsync(h_stats, stats, stats_bytes, hipMemcpyDeviceToHost, s));
+    LF_HIP(hipMemcpyAsync(h_colhist, hist, hist_bytes, hipMemcpyDeviceToHost, s));
+    LF_HIP(hipStreamSynchronize(s));
+    return LF_OK;
+}
+
+size_t lf_hyb_workspace_bytes(int64_t num_rows, int32_t num_parts, int32_t total_buckets) {
+    if (num_rows < 0 || num_parts < 1 || total_buckets < 0) return 0;
+    return hyb_layout(num_rows, num_parts, total_buckets).total;
+}
+
+int lf_hyb_layout(const int64_t* h_ell_rows, const int32_t* h_widths_flat, int32_t total_buckets,
+                  int64_t* h_row_off, int64_t* h_slot_off, int64_t* h_total_rows, int64_t* h_total_slots) {
+    LF_REQUIRE(total_buckets >= 0, LF_ERR_INVALID, "negative bucket count");
+    LF_REQUIRE(h_total_rows && h_total_slots, LF_ERR_INVALID, "null output");
+    LF_REQUIRE(total_buckets == 0 || (h_ell_rows && h_widths_flat && h_row_off && h_slot_off), LF_ERR_INVALID,
+               "null argument");
+    flat_layout(h_ell_rows, h_widths_flat, total_buckets, h_row_off, h_slot_off, h_total_rows, h_total_slots);
+    return LF_OK;
+}
+
+int lf_hyb_plan(const int32_t* d_indptr, const int32_t* d_indices, const int32_t* d_seg_deg,
+                int64_t num_rows, int64_t num_cols, int32_t num_parts, const int32_t* h_widths_flat,
+                const int32_t* h_widths_off, void* d_workspace, size_t workspace_bytes,
+                int64_t* h_ell_rows, lf_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (int rc = check_common(d_indptr, d_indices, num_rows, num_cols, num_parts)) return rc;
+    if (int rc = check_widths(num_parts, h_widths_flat, h_widths_off)) return rc;
+    const int nb = h_widths_off[num_parts];
+    LF_REQUIRE(h_ell_rows || nb == 0, LF_ERR_INVALID, "h_ell_rows is null");
+    const HybLayout L = hyb_layout(num_rows, num_parts, nb);
+    LF_REQUIRE(d_workspace && workspace_bytes >= L.total, LF_ERR_WORKSPACE,
+               "workspace has %zu bytes, %zu needed", workspace_bytes, L.total);
+    char* ws = (char*)d_workspace;
+    int32_t* bnd = (int32_t*)(ws + L.bnd);
+    int32_t* wtab = (int32_t*)(ws + L.wtab);
+    int32_t* flags = (int32_t*)(ws + L.flags);
+    long long* totals = (long long*)(ws + L.totals);
+    int32_t* blockcnt = (int32_t*)(ws + L.blockcnt);
+    const int64_t psize = lf::ceil_div(num_cols, num_parts);
+
+    std::vector<int32_t> h_wtab((size_t)num_parts * kWtabStride, 0);
+    for (int p = 0; p < num_parts; ++p) {
+        const int n = h_widths_off[p + 1] - h_widths_off[p];
+        h_wtab[(size_t)p * kWtabStride] = n;
+        for (int b = 0; b < n; ++b) h_wtab[(size_t)p * kWtabStride + 1 + b] = h_widths_flat[h_widths_off[p] + b];
+        h_wtab[(size_t)p * kWtabStride + 12] = h_widths_off[p];
+    }
+    LF_HIP(hipMemcpyAsync(wtab, h_wtab.data(), h_wtab.size() * 4, hipMemcpyHostToDevice, s));
+    LF_HIP(hipStreamSynchronize(s));     // h_wtab is pageable and about to go out of scope
+    LF_HIP(fill_u32(flags, 64, 0u, s));
+    LF_HIP(fill_u32(totals, (int64_t)std::max(nb, 1) * 2, 0u, s));
+    if (num_rows > 0) {
+        if (num_parts > 1) {
+            seg_bounds_kernel<<<L.nblk, kBlock, 0, s>>>(d_indptr, d_indices, num_rows, num_parts, psize, bnd);
+            LF_HIP(hipGetLastError());
+        }
+        SegView v{d_indptr, bnd, num_rows, num_parts};
+        hyb_count_kernel<<<dim3(L.nblk, num_parts), kBlock, 0, s>>>(v, d_seg_deg, wtab, L.nblk, blockcnt, flags);
+        LF_HIP(hipGetLastError());
+        if (nb > 0) {
+            hyb_scan_kernel<<<nb, 1024, 0, s>>>(blockcnt, L.nblk, totals);
+            LF_HIP(hipGetLastError());
+        }
+    }
+    int32_t h_flags = 0;
+    std::vector<long long> h_tot((size_t)std::max(nb, 1), 0);
+    LF_HIP(hipMemcpyAsync(&h_flags, flags, 4, hipMemcpyDeviceToHost, s));
+    if (nb > 0) LF_HIP(hipMemcpyAsync(h_tot.data(), totals, (size_t)nb * 8, hipMemcpyDeviceToHost, s));
+    LF_HIP(hipStreamSynchronize(s));
+    if (h_flags & 1)
+        return lf::fail(LF_ERR_CONFIG, "list index out of range: a partition with nonzeros has no bucket widths");
+    if (h_flags & 2)
+        return lf::fail(LF_ERR_UNSUPPORTED, "a row is split over more than %d ELL rows", kMetaSegMax);
+    for (int k = 0; k < nb; ++k) h_ell_rows[k] = h_tot[k];
+    return LF_OK;
+}
+
+int lf_hyb_build(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values,
+                 const int32_t* d_seg_deg, int64_t num_rows, int64_t num_cols, int32_t num_parts,
+                 const int32_t* h_widths_flat, const int32_t* h_widths_off, const int64_t* h_ell_rows,
+                 void* d_workspace, size_t workspace_bytes, int32_t* d_rows, int32_t* d_meta,
+                 int32_t* d_cols, float* d_vals, float* d_mask, lf_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (int rc = check_common(d_indptr, d_indices, num_rows, num_cols, num_parts)) return rc;
+    if (int rc = check_widths(num_parts, h_widths_flat, h_widths_off)) return rc;
+    const int nb = h_widths_off[num_parts];
+    if (nb == 0 || num_rows == 0) return LF_OK;
+    LF_REQUIRE(h_ell_rows, LF_ERR_INVALID, "h_ell_rows is null");
+    int64_t total_rows = 0;
+    for (int k = 0; k < nb; ++k) {
+        LF_REQUIRE(h_ell_rows[k] >= 0, LF_ERR_INVALID, "negative ELL row count");
+        total_rows += h_ell_rows[k];
+    }
+    if (total_rows == 0) return LF_OK;
+    LF_REQUIRE(d_rows && d_meta && d_cols && d_vals && d_indices, LF_ERR_INVALID, "slab pointers are null");
+    const HybLayout L = hyb_layout(num_rows, num_parts, nb);
+    LF_REQUIRE(d_workspace && workspace_bytes >= L.total, LF_ERR_WORKSPACE,
+               "workspace has %zu bytes, %zu needed", workspace_bytes, L.total);
+    char* ws = (char*)d_workspace;
+    int32_t* bnd = (int32_t*)(ws + L.bnd);
+    int32_t* wtab = (int32_t*)(ws + L.wtab);
+    long long* row_off = (long long*)(ws + L.row_off);
+    ScatterBucket* scatter = (ScatterBucket*)(ws + L.scatter);
+    int32_t* blockoff = (int32_t*)(ws + L.blockcnt);
+
+    std::vector<long long> h_row_off((size_t)nb);
+    std::vector<ScatterBucket> h_sc((size_t)nb);
+    std::vector<int64_t> roff((size_t)nb), soff((size_t)nb);
+    int64_t flat_rows, flat_slots;
+    flat_layout(h_ell_rows, h_widths_flat, nb, roff.data(), soff.data(), &flat_rows, &flat_slots);
+    std::vector<int> part_of((size_t)nb);
+    for (int p = 0; p < num_parts; ++p)
+        for (int k = h_widths_off[p]; k < h_widths_off[p + 1]; ++k) part_of[k] = p;
+    long long blocks = 0;
+    const long long span = (long long)kBlock * kSlotsPerThread;
+    for (int k = 0; k < nb; ++k) {
+        const int w = h_widths_flat[k];
+        h_row_off[k] = roff[k];
+        h_sc[k].slot_off = soff[k];
+        h_sc[k].row_off = roff[k];
+        h_sc[k].n_slots = (long long)h_ell_rows[k] * w;
+        h_sc[k].log_w = lf::ilog2(w);
+        h_sc[k].block_start = (int)blocks;
+        h_sc[k].part = part_of[k];
+        h_sc[k].pad_ = 0;
+        blocks += (h_sc[k].n_slots + span - 1) / span;
+        LF_REQUIRE(blocks < (1ll << 31), LF_ERR_UNSUPPORTED, "too many slab slots");
+    }
+    LF_HIP(hipMemcpyAsync(row_off, h_row_off.data(), (size_t)nb * 8, hipMemcpyHostToDevice, s));
+    LF_HIP(hipMemcpyAsync(scatter, h_sc.data(), (size_t)nb * sizeof(ScatterBucket), hipMemcpyHostToDevice, s));
+    LF_HIP(hipStreamSynchronize(s));     // pageable sources go out of scope below
+
+    SegView v{d_indptr, bnd, num_rows, num_parts};
+    hyb_rows_kernel<<<dim3(L.nblk, num_parts), kBlock, 0, s>>>(v, d_seg_deg, wtab, L.nblk, blockoff, row_off,
+                                                              d_rows, d_meta);
+    LF_HIP(hipGetLastError());
+    if (blocks > 0) {
+        hyb_scatter_kernel<<<(int)blocks, kBlock, 0, s>>>(scatter, nb, v, d_indices, d_values, d_rows, d_meta,
+                                                         d_cols, d_vals, d_mask);
+        LF_HIP(hipGetLastError());
+    }
+    return LF_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,1022 @@
+// Fused hyb SpMM for gfx950 (MI355X):  C[rows][N] = A_hyb . B[cols][N], fp32 accumulate.
+//
+// Takes over the kernel that the reference generates through SparseTIR/TVM in
+// bench_hyb_with_config (playground_pipline/format_algos.py:388-605): all (partition,
+// bucket) ELL blocks of the hyb format are walked by one launch per column partition.
+// The reference binds 32 threads to 32 features and 8 ELL rows to a thread block and uses
+// atomicAdd where several ELL rows feed one output row (format_algos.py:508-533).  Here:
+//
+//   * a "sub-wave" of LPR lanes owns one ELL row at a time; each lane holds VEC consecutive
+//     features (float4, or 8 x bf16 = 16 bytes), so one B row is read with one 16-byte load
+//     per lane, coalesced along the feature dimension (N = 128 fp32 -> 32 lanes, two rows
+//     per 64-lane wavefront);
+//   * narrow buckets stage their (column, value) tile in LDS with coalesced 16-byte loads
+//     and read it back as broadcasts; wide buckets and the widest bucket of a partition
+//     (whose source rows may span several ELL rows) stream slots through wavefront
+//     shuffles instead;
+//   * a source row split over several ELL rows is summed by one owner; rows longer than
+//     kHeavySlots are cut into chunks, each reduced by a whole workgroup into a partial
+//     row, and a small second kernel adds the partials in fixed order;
+//   * partitions run as consecutive launches: partition 0 stores every output row (rows it
+//     does not touch are cleared by the same launch), later partitions add.  Nothing
+//     depends on scheduling, so results are bit-reproducible, and there are no atomics.
+//
+// The workgroup -> tile mapping is XCD-aware: workgroup i runs on XCD i % 8, and each
+// group of tiles is cut into 8 contiguous ranges, one per XCD, so that neighbouring ELL
+// rows (which tend to share B rows in structured matrices) meet in the same L2.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+#include <vector>
+
+#include "lf_internal.h"
+
+namespace {
+
+constexpr int kWG = 256;            // threads per workgroup (4 wavefronts)
+constexpr int kTileSlots = 2048;    // (col, val) pairs staged in LDS per tile: 16 KiB
+constexpr int kTileRows = 512;      // ELL rows per tile at most
+constexpr int kHeavySlots = 1024;   // a source row with more slab slots is split into chunks
+constexpr int kChunkSlots = 2048;   // slots per chunk (a whole number of ELL rows)
+constexpr int kXcds = 8;
+constexpr int kMaxGroups = 48;      // tile groups per launch
+constexpr int kUnroll = 8;          // B-row gathers in flight per sub-wave
+constexpr uint32_t kMetaLenMask = 0x7FFu;
+constexpr int kMetaLenBits = 11;
+
+enum GroupType : int { kEll = 0, kSeg = 1, kZero = 2, kChunk = 3 };
+
+struct Chunk {
+    long long slot_begin;   // first slot, relative to the bucket's slab
+    int n_slots;
+    int partial;            // index of the partial row this chunk produces
+};
+
+struct HeavyRow {
+    int row;
+    int partial_begin;
+    int n_partials;
+    int pad_;
+};
+
+struct Group {
+    int type;
+    int log_w;
+    int rows_per_tile;
+    int pad_;
+    long long n_items;            // ELL rows / rows to clear / chunks
+    long long n_tiles;
+    const int32_t* rows;          // kEll, kSeg: source rows; kZero: rows to clear
+    const int32_t* meta;
+    const int32_t* cols;
+    const float* vals;
+    const Chunk* chunks;          // kChunk
+};
+
+struct LaunchArgs {
+    const Group* groups;
+    int n_groups;
+    int accumulate;               // 0: C = result, 1: C += result
+    int feat;                     // N
+    int pad_;
+    const void* B;
+    float* C;
+    float* partials;
+};
+
+// ------------------------------------------------------------------------------------
+// Dense-operand access: VEC features per lane as one 16-byte load.
+template <typename BT> struct Dense;
+
+template <> struct Dense<float> {
+    static constexpr int kVec = 4;
+    __device__ static __forceinline__ void load(const void* B, size_t elem, float (&x)[4]) {
+        const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(B) + elem);
+        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    }
+};
+
+struct bf16_t { uint16_t bits; };
+
+template <> struct Dense<bf16_t> {
+    static constexpr int kVec = 8;
+    __device__ static __forceinline__ void load(const void* B, size_t elem, float (&x)[8]) {
+        const uint4 v = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(B) + elem);
+        x[0] = __uint_as_float(v.x << 16); x[1] = __uint_as_float(v.x & 0xFFFF0000u);
+        x[2] = __uint_as_float(v.y << 16); x[3] = __uint_as_float(v.y & 0xFFFF0000u);
+        x[4] = __uint_as_float(v.z << 16); x[5] = __uint_as_float(v.z & 0xFFFF0000u);
+        x[6] = __uint_as_float(v.w << 16); x[7] = __uint_as_float(v.w & 0xFFFF0000u);
+    }
+};
+
+// Accumulator of one sub-wave lane: CH chunks of VEC features.
+template <int CH, int VEC> struct Acc {
+    float v[CH][VEC];
+    __device__ __forceinline__ void clear() {
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) v[c][i] = 0.f;
+    }
+};
+
+// Position of a lane inside the feature dimension.
+template <int LPR, int CH, int VEC> struct Lane {
+    int sl;                 // lane inside the sub-wave
+    int feat;               // N
+    int f[CH];              // first feature of each chunk (clamped to 0 when outside N)
+    bool on[CH];
+    __device__ __forceinline__ Lane(int sl_, int feat_) : sl(sl_), feat(feat_) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int f0 = (c * LPR + sl_) * VEC;
+            on[c] = f0 < feat_;
+            f[c] = on[c] ? f0 : 0;
+        }
+    }
+};
+
+template <int LPR, int CH, typename BT>
+__device__ __forceinline__ void gather_fma(const void* B, const Lane<LPR, CH, Dense<BT>::kVec>& ln,
+                                           const int (&col)[kUnroll], const float (&val)[kUnroll],
+                                           Acc<CH, Dense<BT>::kVec>& acc) {
+    constexpr int VEC = Dense<BT>::kVec;
+    float x[kUnroll][CH][VEC];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+            Dense<BT>::load(B, (size_t)(uint32_t)col[u] * (size_t)ln.feat + ln.f[c], x[u][c]);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc.v[c][i] = fmaf(val[u], x[u][c][i], acc.v[c][i]);
+}
+
+template <int LPR, int CH, int VEC>
+__device__ __forceinline__ void store_row(float* C, int row, const Lane<LPR, CH, VEC>& ln,
+                                          const Acc<CH, VEC>& acc, int accumulate) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        if (!ln.on[c]) continue;
+        float* dst = C + (size_t)row * ln.feat + ln.f[c];
+#pragma unroll
+        for (int i = 0; i < VEC; i += 4) {
+            float4 o = make_float4(acc.v[c][i], acc.v[c][i + 1], acc.v[c][i + 2], acc.v[c][i + 3]);
+            if (accumulate) {
+                const float4 old = *reinterpret_cast<const float4*>(dst + i);
+                o.x += old.x; o.y += old.y; o.z += old.z; o.w += old.w;
+            }
+            *reinterpret_cast<float4*>(dst + i) = o;
+        }
+    }
+}
+
+// Sum of `total` consecutive slab slots starting at `base`, streamed by one sub-wave: each
+// lane loads one (col, val), the sub-wave then walks them by shuffle.  Slots past `total`
+// are replaced by (first column, 0) so that every gather is unconditional and in range.
+template <int LPR, int CH, typename BT>
+__device__ __forceinline__ void stream_slots(const int32_t* __restrict__ cols, const float* __restrict__ vals,
+                                             long long base, int total, const void* B,
+                                             const Lane<LPR, CH, Dense<BT>::kVec>& ln,
+                                             Acc<CH, Dense<BT>::kVec>& acc) {
+    if (total <= 0) return;
+    const int c_first = cols[base];
+    for (int off = 0; off < total; off += LPR) {
+        const int idx = off + ln.sl;
+        const bool have = idx < total;
+        const int my_c = have ? cols[base + idx] : c_first;
+        const float my_v = have ? (vals ? vals[base + idx] : 1.f) : 0.f;
+        const int cnt = min(LPR, total - off);
+        for (int j = 0; j < cnt; j += kUnroll) {
+            int c[kUnroll];
+            float v[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                c[u] = __shfl(my_c, j + u, LPR);
+                v[u] = __shfl(my_v, j + u, LPR);
+            }
+            gather_fma<LPR, CH, BT>(B, ln, c, v, acc);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// Tile bodies.  `smem` is the workgroup's LDS: kTileSlots int2 pairs followed by
+// kTileRows int2 (row, meta) entries.
+
+// Narrow bucket: W slots per ELL row, rows independent (one ELL row per source row).
+// RPI rows are processed together by a sub-wave so that kUnroll gathers are in flight
+// even when W < kUnroll.
+template <int W, int LPR, int CH, typename BT>
+__device__ __forceinline__ void ell_tile_narrow(const int2* s_pairs, const int2* s_rm, int n,
+                                                const LaunchArgs& a, int sw, int sl) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int SW = kWG / LPR;
+    constexpr int RPI = kUnroll / W;
+    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    for (int r0 = sw * RPI; r0 < n; r0 += SW * RPI) {
+        Acc<CH, VEC> acc[RPI];
+        int c[kUnroll];
+        float v[kUnroll];
+#pragma unroll
+        for (int q = 0; q < RPI; ++q) {
+            acc[q].clear();
+            const int r = min(r0 + q, n - 1);
+            const int len = s_rm[r].y & kMetaLenMask;
+            const int c0 = s_pairs[r * W].x;
+#pragma unroll
+            for (int j = 0; j < W; ++j) {
+                const int2 cv = s_pairs[r * W + j];
+                c[q * W + j] = j < len ? cv.x : c0;
+                v[q * W + j] = __int_as_float(cv.y);
+            }
+        }
+        {
+            float x[kUnroll][CH][VEC];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                for (int cc = 0; cc < CH; ++cc)
+                    Dense<BT>::load(a.B, (size_t)(uint32_t)c[u] * (size_t)ln.feat + ln.f[cc], x[u][cc]);
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                for (int cc = 0; cc < CH; ++cc)
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i)
+                        acc[u / W].v[cc][i] = fmaf(v[u], x[u][cc][i], acc[u / W].v[cc][i]);
+        }
+#pragma unroll
+        for (int q = 0; q < RPI; ++q)
+            if (r0 + q < n) store_row<LPR, CH, VEC>(a.C, s_rm[r0 + q].x, ln, acc[q], a.accumulate);
+    }
+}
+
+// Bucket with W >= kUnroll staged in LDS: one ELL row per sub-wave at a time.
+template <int LPR, int CH, typename BT>
+__device__ __forceinline__ void ell_tile_wide(const int2* s_pairs, const int2* s_rm, int n, int log_w,
+                                              const LaunchArgs& a, int sw, int sl) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int SW = kWG / LPR;
+    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    for (int r = sw; r < n; r += SW) {
+        const int2 rm = s_rm[r];
+        const int len = rm.y & kMetaLenMask;
+        const int2* rp = s_pairs + (r << log_w);
+        const int c0 = rp[0].x;
+        Acc<CH, VEC> acc;
+        acc.clear();
+        for (int j = 0; j < len; j += kUnroll) {
+            int c[kUnroll];
+            float v[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const int2 cv = rp[j + u];
+                c[u] = j + u < len ? cv.x : c0;
+                v[u] = __int_as_float(cv.y);
+            }
+            gather_fma<LPR, CH, BT>(a.B, ln, c, v, acc);
+        }
+        store_row<LPR, CH, VEC>(a.C, rm.x, ln, acc, a.accumulate);
+    }
+}
+
+template <int LPR, int CH, typename BT>
+__device__ __forceinline__ void run_ell_tile(const Group& g, long long tile, int2* s_pairs, int2* s_rm,
+                                             const LaunchArgs& a) {
+    const int tid = threadIdx.x;
+    const long long e0 = tile * g.rows_per_tile;
+    const int n = (int)min((long long)g.rows_per_tile, g.n_items - e0);
+    const int n_slots = n << g.log_w;
+    const long long s0 = e0 << g.log_w;
+    __syncthreads();                       // LDS of the previous tile is no longer read
+    for (int i = tid * 4; i < n_slots; i += kWG * 4) {
+        if (i + 4 <= n_slots) {            // s0 and i are multiples of 4, slabs are 16-byte aligned
+            const int4 c = *reinterpret_cast<const int4*>(g.cols + s0 + i);
+            const int4 v = *reinterpret_cast<const int4*>(g.vals + s0 + i);
+            s_pairs[i + 0] = make_int2(c.x, v.x);
+            s_pairs[i + 1] = make_int2(c.y, v.y);
+            s_pairs[i + 2] = make_int2(c.z, v.z);
+            s_pairs[i + 3] = make_int2(c.w, v.w);
+        } else {
+            for (int k = i; k < n_slots; ++k)
+                s_pairs[k] = make_int2(g.cols[s0 + k], __float_as_int(g.vals[s0 + k]));
+        }
+    }
+    for (int i = tid; i < n; i += kWG) s_rm[i] = make_int2(g.rows[e0 + i], g.meta[e0 + i]);
+    __syncthreads();
+    const int sw = tid / LPR, sl = tid % LPR;
+    switch (g.log_w) {
+        case 0: ell_tile_narrow<1, LPR, CH, BT>(s_pairs, s_rm, n, a, sw, sl); break;
+        case 1: ell_tile_narrow<2, LPR, CH, BT>(s_pairs, s_rm, n, a, sw, sl); break;
+        case 2: ell_tile_narrow<4, LPR, CH, BT>(s_pairs, s_rm, n, a, sw, sl); break;
+        default: ell_tile_wide<LPR, CH, BT>(s_pairs, s_rm, n, g.log_w, a, sw, sl); break;
+    }
+}
+
+// Bucket whose source rows may span several ELL rows, or whose rows are too wide to stage:
+// the first ELL row of a segment owns it and streams all of its slots; continuation rows
+// and segments above kHeavySlots (handled as chunks) are skipped.
+template <int LPR, int CH, typename BT>
+__device__ __forceinline__ void run_seg_tile(const Group& g, long long tile, const LaunchArgs& a) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int SW = kWG / LPR;
+    const int tid = threadIdx.x;
+    const int sw = tid / LPR, sl = tid % LPR;
+    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const long long e0 = tile * g.rows_per_tile;
+    const int n = (int)min((long long)g.rows_per_tile, g.n_items - e0);
+    for (int r = sw; r < n; r += SW) {
+        const long long e = e0 + r;
+        const int m = g.meta[e];
+        if (m < 0) continue;                                   // continuation row
+        const int seg = (int)((uint32_t)m >> kMetaLenBits);
+        if (((long long)seg << g.log_w) > kHeavySlots) continue;
+        int total = m & kMetaLenMask;
+        if (seg > 1) total = ((seg - 1) << g.log_w) + (g.meta[e + seg - 1] & kMetaLenMask);
+        Acc<CH, VEC> acc;
+        acc.clear();
+        stream_slots<LPR, CH, BT>(g.cols, g.vals, e << g.log_w, total, a.B, ln, acc);
+        store_row<LPR, CH, VEC>(a.C, g.rows[e], ln, acc, a.accumulate);
+    }
+}
+
+template <int LPR, int CH, typename BT>
+__device__ __forceinline__ void run_zero_tile(const Group& g, long long tile, const LaunchArgs& a) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int SW = kWG / LPR;
+    const int tid = threadIdx.x;
+    const int sw = tid / LPR, sl = tid % LPR;
+    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const long long e0 = tile * g.rows_per_tile;
+    const int n = (int)min((long long)g.rows_per_tile, g.n_items - e0);
+    Acc<CH, VEC> zero;
+    zero.clear();
+    for (int r = sw; r < n; r += SW) store_row<LPR, CH, VEC>(a.C, g.rows[e0 + r], ln, zero, 0);
+}
+
+// One chunk of a heavy source row: the workgroup's sub-waves take consecutive slices of
+// the chunk, their sums are combined through LDS in sub-wave order.
+template <int LPR, int CH, typename BT>
+__device__ __forceinline__ void run_chunk_tile(const Group& g, long long tile, float* s_red,
+                                               const LaunchArgs& a) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int SW = kWG / LPR;
+    const int tid = threadIdx.x;
+    const int sw = tid / LPR, sl = tid % LPR;
+    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const Chunk ck = g.chunks[tile];
+    int per = (ck.n_slots + SW - 1) / SW;
+    per = (per + LPR - 1) / LPR * LPR;
+    const int lo = min(sw * per, ck.n_slots);
+    const int hi = min(lo + per, ck.n_slots);
+    Acc<CH, VEC> acc;
+    acc.clear();
+    stream_slots<LPR, CH, BT>(g.cols, g.vals, ck.slot_begin + lo, hi - lo, a.B, ln, acc);
+    __syncthreads();                       // LDS of the previous tile is no longer read
+    // s_red[sw][c][sl][i]
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) s_red[((sw * CH + c) * LPR + sl) * VEC + i] = acc.v[c][i];
+    __syncthreads();
+    if (sw == 0) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            if (!ln.on[c]) continue;
+            float sum[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) sum[i] = 0.f;
+            for (int s = 0; s < SW; ++s)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) sum[i] += s_red[((s * CH + c) * LPR + sl) * VEC + i];
+            float* dst = a.partials + (size_t)ck.partial * a.feat + ln.f[c];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) dst[i] = sum[i];
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// The fused kernel: a persistent grid walks all tile groups of one column partition.
+template <int LPR, int CH, typename BT>
+__global__ void __launch_bounds__(kWG)
+spmm_partition_kernel(LaunchArgs a) {
+    __shared__ int2 s_pairs[kTileSlots];
+    __shared__ int2 s_rm[kTileRows];
+    __shared__ Group s_groups[kMaxGroups];
+
+    {   // the group table is small: copy it into LDS once
+        const int words = a.n_groups * (int)(sizeof(Group) / 4);
+        const int32_t* src = reinterpret_cast<const int32_t*>(a.groups);
+        int32_t* dst = reinterpret_cast<int32_t*>(s_groups);
+        for (int i = threadIdx.x; i < words; i += kWG) dst[i] = src[i];
+    }
+    __syncthreads();
+
+    const int xcd = blockIdx.x % kXcds;
+    const int local = blockIdx.x / kXcds;
+    const int per_xcd = gridDim.x / kXcds;
+
+    // This XCD's share of group g is tiles [n*xcd/8, n*(xcd+1)/8); the shares of all groups
+    // are concatenated and dealt to the XCD's workgroups round-robin.
+    long long v = local;           // position in the concatenated list
+    long long skipped = 0;         // list positions before the current group
+    for (int gi = 0; gi < a.n_groups; ++gi) {
+        const Group& g = s_groups[gi];
+        const long long lo = g.n_tiles * xcd / kXcds;
+        const long long hi = g.n_tiles * (xcd + 1) / kXcds;
+        const long long cnt = hi - lo;
+        while (v - skipped < cnt) {
+            const long long tile = lo + (v - skipped);
+            switch (g.type) {
+                case kEll: run_ell_tile<LPR, CH, BT>(g, tile, s_pairs, s_rm, a); break;
+                case kSeg: run_seg_tile<LPR, CH, BT>(g, tile, a); break;
+                case kZero: run_zero_tile<LPR, CH, BT>(g, tile, a); break;
+                default: run_chunk_tile<LPR, CH, BT>(g, tile, reinterpret_cast<float*>(s_pairs), a); break;
+            }
+            v += per_xcd;
+        }
+        skipped += cnt;
+    }
+}
+
+// Adds the partial rows of every heavy source row in chunk order and writes the row.
+template <int LPR, int CH, typename BT>
+__global__ void __launch_bounds__(kWG)
+spmm_finalize_kernel(const HeavyRow* __restrict__ heavy, int n_heavy, LaunchArgs a) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int SW = kWG / LPR;
+    const int sw = threadIdx.x / LPR, sl = threadIdx.x % LPR;
+    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    for (int h = blockIdx.x * SW + sw; h < n_heavy; h += gridDim.x * SW) {
+        const HeavyRow hr = heavy[h];
+        Acc<CH, VEC> acc;
+        acc.clear();
+        for (int k = 0; k < hr.n_partials; ++k) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                if (!ln.on[c]) continue;
+                const float* src = a.partials + (size_t)(hr.partial_begin + k) * a.feat + ln.f[c];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc.v[c][i] += src[i];
+            }
+        }
+        store_row<LPR, CH, VEC>(a.C, hr.row, ln, acc, a.accumulate);
+    }
+}
+
+// Row-parallel CSR product: one sub-wave per row, entries streamed by shuffle.
+template <int LPR, int CH, typename BT>
+__global__ void __launch_bounds__(kWG)
+csr_spmm_kernel(const int32_t* __restrict__ indptr, const int32_t* __restrict__ indices,
+                const float* __restrict__ values, long long n_rows, LaunchArgs a) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int SW = kWG / LPR;
+    const int sw = threadIdx.x / LPR, sl = threadIdx.x % LPR;
+    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    for (long long r = (long long)blockIdx.x * SW + sw; r < n_rows; r += (long long)gridDim.x * SW) {
+        const int lo = indptr[r], hi = indptr[r + 1];
+        Acc<CH, VEC> acc;
+        acc.clear();
+        stream_slots<LPR, CH, BT>(indices, values, lo, hi - lo, a.B, ln, acc);
+        store_row<LPR, CH, VEC>(a.C, (int)r, ln, acc, 0);
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// Plan-time kernels.
+
+// meta from rows / vals for slabs that come without one: len = position of the last
+// nonzero value + 1 (at least 1); segment counts from runs of equal row ids.
+__global__ void derive_meta_kernel(const int32_t* __restrict__ rows, const float* __restrict__ vals,
+                                   long long n_rows, int log_w, int32_t* __restrict__ meta) {
+    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n_rows) return;
+    const int w = 1 << log_w;
+    const float* rv = vals + (e << log_w);
+    int len = 1;
+    for (int j = w - 1; j > 0; --j)
+        if (rv[j] != 0.f) { len = j + 1; break; }
+    const int r = rows[e];
+    uint32_t field, cont = 0;
+    if (e > 0 && rows[e - 1] == r) {
+        long long h = e - 1;
+        while (h > 0 && rows[h - 1] == r) --h;
+        field = (uint32_t)(e - h);
+        cont = 0x80000000u;
+    } else {
+        long long t = e + 1;
+        while (t < n_rows && rows[t] == r) ++t;
+        field = (uint32_t)(t - e);
+    }
+    meta[e] = (int32_t)((uint32_t)len | (field << kMetaLenBits) | cont);
+}
+
+// Per bucket: does any ELL row belong to a multi-row segment; list of heavy segment heads.
+__global__ void scan_meta_kernel(const int32_t* __restrict__ meta, long long n_rows, int log_w,
+                                 int* __restrict__ flag_multi, int* __restrict__ heavy_count,
+                                 long long* __restrict__ heavy_list, int heavy_cap) {
+    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n_rows) return;
+    const int m = meta[e];
+    if (m < 0) { *flag_multi = 1; return; }
+    const int seg = (int)((uint32_t)m >> kMetaLenBits);
+    if (seg > 1) *flag_multi = 1;
+    if (((long long)seg << log_w) > kHeavySlots) {
+        const int at = atomicAdd(heavy_count, 1);
+        if (at < heavy_cap) heavy_list[at] = e;
+    }
+}
+
+__global__ void mark_rows_kernel(const int32_t* __restrict__ rows, long long n, uint8_t* __restrict__ covered) {
+    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < n) covered[rows[e]] = 1;
+}
+
+__global__ void collect_uncovered_kernel(const uint8_t* __restrict__ covered, long long n_rows,
+                                         int* __restrict__ count, int32_t* __restrict__ list) {
+    const long long r = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= n_rows || covered[r]) return;
+    const int at = atomicAdd(count, 1);
+    if (list) list[at] = (int32_t)r;
+}
+
+__global__ void fill_bytes_kernel(uint32_t* __restrict__ p, long long n_words, uint32_t value) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n_words;
+         i += (long long)gridDim.x * blockDim.x)
+        p[i] = value;
+}
+
+}  // namespace
+
+// ====================================================================================
+struct lf_spmm_plan {
+    int feat = 0, b_dtype = 0, num_parts = 0;
+    int64_t num_rows = 0, num_cols = 0;
+    int lpr = 0, ch = 0;
+    int device = 0, num_cus = 0, grid = 0;
+    struct Launch {
+        int group_begin = 0, n_groups = 0;
+        long long tiles = 0;
+        int heavy_begin = 0, n_heavy = 0;
+    };
+    std::vector<Launch> launches;
+    std::vector<void*> owned;        // device allocations released by destroy
+    Group* d_groups = nullptr;
+    HeavyRow* d_heavy = nullptr;
+    float* d_partials = nullptr;
+    int64_t info[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+};
+
+namespace {
+
+template <typename T> int dev_alloc(lf_spmm_plan* p, T** out, size_t count) {
+    *out = nullptr;
+    if (count == 0) return LF_OK;
+    void* ptr = nullptr;
+    LF_HIP(hipMalloc(&ptr, count * sizeof(T)));
+    p->owned.push_back(ptr);
+    *out = (T*)ptr;
+    return LF_OK;
+}
+
+using KernelFn = void (*)(LaunchArgs);
+using FinalFn = void (*)(const HeavyRow*, int, LaunchArgs);
+using CsrFn = void (*)(const int32_t*, const int32_t*, const float*, long long, LaunchArgs);
+
+struct KernelSet {
+    KernelFn tiles = nullptr;
+    FinalFn finalize = nullptr;
+    CsrFn csr = nullptr;
+};
+
+template <int LPR, int CH> void pick_kernels(int dtype, KernelSet* k) {
+    if (dtype == LF_DTYPE_BF16) {
+        k->tiles = spmm_partition_kernel<LPR, CH, bf16_t>;
+        k->finalize = spmm_finalize_kernel<LPR, CH, bf16_t>;
+        k->csr = csr_spmm_kernel<LPR, CH, bf16_t>;
+    } else {
+        k->tiles = spmm_partition_kernel<LPR, CH, float>;
+        k->finalize = spmm_finalize_kernel<LPR, CH, float>;
+        k->csr = csr_spmm_kernel<LPR, CH, float>;
+    }
+}
+
+int select_kernels(int lpr, int ch, int dtype, KernelSet* k) {
+    if (ch == 1) {
+        switch (lpr) {
+            case 8: pick_kernels<8, 1>(dtype, k); break;
+            case 16: pick_kernels<16, 1>(dtype, k); break;
+            case 32: pick_kernels<32, 1>(dtype, k); break;
+            case 64: pick_kernels<64, 1>(dtype, k); break;
+        }
+    } else if (lpr == 64 && ch == 2) {
+        pick_kernels<64, 2>(dtype, k);
+    } else if (lpr == 64 && ch == 4) {
+        pick_kernels<64, 4>(dtype, k);
+    }
+    LF_REQUIRE(k->tiles != nullptr, LF_ERR_UNSUPPORTED, "no kernel for %d lanes x %d chunks", lpr, ch);
+    return LF_OK;
+}
+
+int feature_shape(int feat, int dtype, int* lpr, int* ch) {
+    const int vec = dtype == LF_DTYPE_BF16 ? 8 : 4;
+    LF_REQUIRE(feat >= 32 && feat % 32 == 0, LF_ERR_UNSUPPORTED,
+               "feat_size must be a positive multiple of 32 (got %d)", feat);
+    LF_REQUIRE(feat <= 1024, LF_ERR_UNSUPPORTED, "feat_size above 1024 is not supported (got %d)", feat);
+    const int lanes = feat / vec;
+    int l = 8;
+    while (l < lanes && l < 64) l <<= 1;
+    int c = (lanes + l - 1) / l;
+    if (c == 3) c = 4;
+    LF_REQUIRE(c == 1 || c == 2 || c == 4, LF_ERR_UNSUPPORTED, "feat_size %d is not supported", feat);
+    *lpr = l;
+    *ch = c;
+    return LF_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int lf_spmm_destroy(lf_spmm_plan* plan) {
+    if (!plan) return LF_OK;
+    int rc = LF_OK;
+    for (void* p : plan->owned)
+        if (hipFree(p) != hipSuccess) rc = LF_ERR_HIP;
+    delete plan;
+    if (rc != LF_OK) return lf::fail(rc, "hipFree failed while destroying the plan");
+    return LF_OK;
+}
+
+int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int32_t num_buckets,
+                   int32_t num_parts, int64_t num_rows, int64_t num_cols, int32_t feat_size,
+                   int32_t b_dtype, lf_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    LF_REQUIRE(out_plan, LF_ERR_INVALID, "out_plan is null");
+    *out_plan = nullptr;
+    LF_REQUIRE(num_buckets >= 0 && (num_buckets == 0 || h_buckets), LF_ERR_INVALID, "bucket list is null");
+    LF_REQUIRE(num_parts >= 1, LF_ERR_INVALID, "num_parts must be >= 1");
+    LF_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31) && num_cols >= 1 && num_cols < (1ll << 31),
+               LF_ERR_INVALID, "bad shape");
+    LF_REQUIRE(b_dtype == LF_DTYPE_F32 || b_dtype == LF_DTYPE_BF16, LF_ERR_INVALID, "unknown B dtype %d", b_dtype);
+    int lpr, ch;
+    if (int rc = feature_shape(feat_size, b_dtype, &lpr, &ch)) return rc;
+    const int sw = kWG / lpr;
+    for (int k = 0; k < num_buckets; ++k) {
+        const lf_bucket_desc& b = h_buckets[k];
+        LF_REQUIRE(lf::is_pow2(b.width) && b.width <= 1024, LF_ERR_INVALID, "bucket %d: width %d", k, b.width);
+        LF_REQUIRE(b.part >= 0 && b.part < num_parts, LF_ERR_INVALID, "bucket %d: partition %d", k, b.part);
+        LF_REQUIRE(b.num_ell_rows >= 0 && b.num_ell_rows < (1ll << 31), LF_ERR_INVALID, "bucket %d: row count", k);
+        LF_REQUIRE(k == 0 || h_buckets[k - 1].part <= b.part, LF_ERR_INVALID, "buckets must be ordered by partition");
+        if (b.num_ell_rows > 0) {
+            LF_REQUIRE(b.d_rows && b.d_cols && b.d_vals, LF_ERR_INVALID, "bucket %d: null slab", k);
+            LF_REQUIRE(((uintptr_t)b.d_cols % 16 == 0) && ((uintptr_t)b.d_vals % 16 == 0), LF_ERR_INVALID,
+                       "bucket %d: slabs must be 16-byte aligned", k);
+        }
+    }
+
+    lf_spmm_plan* plan = new lf_spmm_plan();
+    plan->feat = feat_size;
+    plan->b_dtype = b_dtype;
+    plan->num_parts = num_parts;
+    plan->num_rows = num_rows;
+    plan->num_cols = num_cols;
+    plan->lpr = lpr;
+    plan->ch = ch;
+    auto bail = [&](int rc) {
+        std::string keep = lf::last_error();
+        lf_spmm_destroy(plan);
+        lf::last_error() = keep;
+        return rc;
+    };
+#define LF_TRY(expr)                        \
+    do {                                    \
+        int _rc = (expr);                   \
+        if (_rc != LF_OK) return bail(_rc); \
+    } while (0)
+#define LF_TRY_HIP(call)                                                                          \
+    do {                                                                                          \
+        hipError_t _e = (call);                                                                   \
+        if (_e != hipSuccess)                                                                     \
+            return bail(lf::fail(LF_ERR_HIP, "%s failed: %s", #call, hipGetErrorString(_e)));     \
+    } while (0)
+
+    hipDeviceProp_t prop;
+    LF_TRY_HIP(hipGetDevice(&plan->device));
+    LF_TRY_HIP(hipGetDeviceProperties(&prop, plan->device));
+    plan->num_cus = prop.multiProcessorCount;
+
+    // ---- meta: derive where missing; classify buckets; collect heavy segments
+    std::vector<const int32_t*> meta((size_t)num_buckets, nullptr);
+    int* d_counters = nullptr;              // [0] multi flag, [1] heavy count, [2] uncovered count
+    LF_TRY(dev_alloc(plan, &d_counters, 4));
+    std::vector<int> is_multi((size_t)num_buckets, 0);
+    std::vector<std::vector<long long>> heavy_heads((size_t)num_buckets);
+    for (int k = 0; k < num_buckets; ++k) {
+        const lf_bucket_desc& b = h_buckets[k];
+        if (b.num_ell_rows == 0) continue;
+        const int log_w = lf::ilog2(b.width);
+        const int grid = (int)((b.num_ell_rows + 255) / 256);
+        if (b.d_meta) {
+            meta[k] = b.d_meta;
+        } else {
+            int32_t* m = nullptr;
+            LF_TRY(dev_alloc(plan, &m, (size_t)b.num_ell_rows));
+            derive_meta_kernel<<<grid, 256, 0, s>>>(b.d_rows, b.d_vals, b.num_ell_rows, log_w, m);
+            LF_TRY_HIP(hipGetLastError());
+            meta[k] = m;
+        }
+        // a heavy segment has more than kHeavySlots slots, so there are fewer than slots / kHeavySlots
+        const long long cap = (b.num_ell_rows << log_w) / kHeavySlots + 1;
+        long long* d_list = nullptr;
+        LF_TRY_HIP(hipMalloc((void**)&d_list, (size_t)cap * 8));
+        fill_bytes_kernel<<<1, 64, 0, s>>>((uint32_t*)d_counters, 4, 0u);
+        scan_meta_kernel<<<grid, 256, 0, s>>>(meta[k], b.num_ell_rows, log_w, d_counters, d_counters + 1,
+                                              d_list, (int)cap);
+        int h_cnt[2] = {0, 0};
+        hipError_t e1 = hipGetLastError();
+        if (e1 == hipSuccess) e1 = hipMemcpyAsync(h_cnt, d_counters, 8, hipMemcpyDeviceToHost, s);
+        if (e1 == hipSuccess) e1 = hipStreamSynchronize(s);
+        if (e1 == hipSuccess && h_cnt[1] > 0) {
+            heavy_heads[k].resize((size_t)h_cnt[1]);
+            e1 = hipMemcpy(heavy_heads[k].data(), d_list, (size_t)h_cnt[1] * 8, hipMemcpyDeviceToHost);
+        }
+        hipError_t e2 = hipFree(d_list);
+        LF_TRY_HIP(e1);
+        LF_TRY_HIP(e2);
+        is_multi[k] = h_cnt[0];
+        std::sort(heavy_heads[k].begin(), heavy_heads[k].end());
+    }
+
+    // ---- chunks and partial rows of heavy segments (host; their number is small)
+    std::vector<std::vector<Chunk>> chunks((size_t)num_buckets);
+    std::vector<HeavyRow> heavy_rows;
+    std::vector<int> heavy_part;
+    int n_partials = 0;
+    for (int k = 0; k < num_buckets; ++k) {
+        if (heavy_heads[k].empty()) continue;
+        const lf_bucket_desc& b = h_buckets[k];
+        const int log_w = lf::ilog2(b.width);
+        // the head's meta gives the ELL-row count; the valid length of the last ELL row and the
+        // source row id are read back
+        std::vector<int32_t> head_meta(heavy_heads[k].size()), last_meta(heavy_heads[k].size()),
+            head_row(heavy_heads[k].size());
+        for (size_t i = 0; i < heavy_heads[k].size(); ++i) {
+            const long long e = heavy_heads[k][i];
+            LF_TRY_HIP(hipMemcpy(&head_meta[i], meta[k] + e, 4, hipMemcpyDeviceToHost));
+            const int seg = (int)((uint32_t)head_meta[i] >> kMetaLenBits);
+            LF_TRY_HIP(hipMemcpy(&last_meta[i], meta[k] + e + seg - 1, 4, hipMemcpyDeviceToHost));
+            LF_TRY_HIP(hipMemcpy(&head_row[i], b.d_rows + e, 4, hipMemcpyDeviceToHost));
+        }
+        const int rows_per_chunk = std::max(1, kChunkSlots >> log_w);
+        for (size_t i = 0; i < heavy_heads[k].size(); ++i) {
+            const long long e = heavy_heads[k][i];
+            const int seg = (int)((uint32_t)head_meta[i] >> kMetaLenBits);
+            const long long total = ((long long)(seg - 1) << log_w) + (last_meta[i] & kMetaLenMask);
+            HeavyRow hr{head_row[i], n_partials, 0, 0};
+            for (int r0 = 0; r0 < seg; r0 += rows_per_chunk) {
+                const long long lo = (long long)r0 << log_w;
+                const long long hi = std::min<long long>(total, (long long)(r0 + rows_per_chunk) << log_w);
+                chunks[k].push_back(Chunk{(e << log_w) + lo, (int)(hi - lo), n_partials});
+                ++n_partials;
+                ++hr.n_partials;
+            }
+            heavy_rows.push_back(hr);
+            heavy_part.push_back(b.part);
+        }
+    }
+    // heavy rows grouped by partition (buckets are ordered by partition already)
+    if (!heavy_rows.empty()) {
+        LF_TRY(dev_alloc(plan, &plan->d_heavy, heavy_rows.size()));
+        LF_TRY_HIP(hipMemcpy(plan->d_heavy, heavy_rows.data(), heavy_rows.size() * sizeof(HeavyRow), hipMemcpyHostToDevice));
+        LF_TRY(dev_alloc(plan, &plan->d_partials, (size_t)n_partials * feat_size));
+    }
+
+    // ---- rows that partition 0 does not write are cleared by its launch
+    int32_t* d_zero_rows = nullptr;
+    int n_zero = 0;
+    if (num_rows > 0) {
+        uint8_t* d_cov = nullptr;
+        const size_t cov_words = ((size_t)num_rows + 3) / 4;
+        LF_TRY_HIP(hipMalloc((void**)&d_cov, cov_words * 4));
+        hipError_t e = hipSuccess;
+        fill_bytes_kernel<<<(int)std::min<size_t>((cov_words + 255) / 256, 4096), 256, 0, s>>>((uint32_t*)d_cov, (long long)cov_words, 0u);
+        for (int k = 0; k < num_buckets && e == hipSuccess; ++k) {
+            const lf_bucket_desc& b = h_buckets[k];
+            if (b.part != 0 || b.num_ell_rows == 0) continue;
+            mark_rows_kernel<<<(int)((b.num_ell_rows + 255) / 256), 256, 0, s>>>(b.d_rows, b.num_ell_rows, d_cov);
+            e = hipGetLastError();
+        }
+        const int rgrid = (int)((num_rows + 255) / 256);
+        if (e == hipSuccess) {
+            fill_bytes_kernel<<<1, 64, 0, s>>>((uint32_t*)d_counters, 4, 0u);
+            collect_uncovered_kernel<<<rgrid, 256, 0, s>>>(d_cov, num_rows, d_counters + 2, nullptr);
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess) e = hipMemcpyAsync(&n_zero, d_counters + 2, 4, hipMemcpyDeviceToHost, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+        if (e == hipSuccess && n_zero > 0) {
+            int rc = dev_alloc(plan, &d_zero_rows, (size_t)n_zero);
+            if (rc != LF_OK) { hipFree(d_cov); return bail(rc); }
+            fill_bytes_kernel<<<1, 64, 0, s>>>((uint32_t*)d_counters, 4, 0u);
+            collect_uncovered_kernel<<<rgrid, 256, 0, s>>>(d_cov, num_rows, d_counters + 2, d_zero_rows);
+            e = hipGetLastError();
+            if (e == hipSuccess) e = hipStreamSynchronize(s);
+        }
+        hipError_t e2 = hipFree(d_cov);
+        LF_TRY_HIP(e);
+        LF_TRY_HIP(e2);
+    }
+
+    // ---- tile groups per launch: chunks first (longest), then buckets widest first, then clears
+    std::vector<Group> groups;
+    std::vector<Chunk*> d_chunks((size_t)num_buckets, nullptr);
+    for (int k = 0; k < num_buckets; ++k) {
+        if (chunks[k].empty()) continue;
+        LF_TRY(dev_alloc(plan, &d_chunks[k], chunks[k].size()));
+        LF_TRY_HIP(hipMemcpy(d_chunks[k], chunks[k].data(), chunks[k].size() * sizeof(Chunk), hipMemcpyHostToDevice));
+    }
+    plan->launches.resize((size_t)num_parts);
+    size_t heavy_cursor = 0;
+    long long total_tiles = 0;
+    for (int p = 0; p < num_parts; ++p) {
+        lf_spmm_plan::Launch& L = plan->launches[p];
+        L.group_begin = (int)groups.size();
+        L.heavy_begin = (int)heavy_cursor;
+        while (heavy_cursor < heavy_rows.size() && heavy_part[heavy_cursor] == p) ++heavy_cursor;
+        L.n_heavy = (int)heavy_cursor - L.heavy_begin;
+        std::vector<int> mine;
+        for (int k = 0; k < num_buckets; ++k)
+            if (h_buckets[k].part == p && h_buckets[k].num_ell_rows > 0) mine.push_back(k);
+        for (int k : mine) {
+            if (chunks[k].empty()) continue;
+            Group g{};
+            g.type = kChunk;
+            g.log_w = lf::ilog2(h_buckets[k].width);
+            g.rows_per_tile = 1;
+            g.n_items = g.n_tiles = (long long)chunks[k].size();
+            g.cols = h_buckets[k].d_cols;
+            g.vals = h_buckets[k].d_vals;
+            g.chunks = d_chunks[k];
+            groups.push_back(g);
+        }
+        std::sort(mine.begin(), mine.end(), [&](int x, int y) { return h_buckets[x].width > h_buckets[y].width; });
+        for (int k : mine) {
+            const lf_bucket_desc& b = h_buckets[k];
+            Group g{};
+            g.log_w = lf::ilog2(b.width);
+            const int fit = kTileSlots >> g.log_w;          // ELL rows whose slots fit the LDS tile
+            const bool staged = !is_multi[k] && fit >= sw;
+            g.type = staged ? kEll : kSeg;
+            g.rows_per_tile = staged ? std::min(kTileRows, fit) : std::max(sw, fit);
+            g.n_items = b.num_ell_rows;
+            g.n_tiles = lf::ceil_div(g.n_items, g.rows_per_tile);
+            g.rows = b.d_rows;
+            g.meta = meta[k];
+            g.cols = b.d_cols;
+            g.vals = b.d_vals;
+            groups.push_back(g);
+        }
+        if (p == 0 && n_zero > 0) {
+            Group g{};
+            g.type = kZero;
+            g.rows_per_tile = 1024;
+            g.n_items = n_zero;
+            g.n_tiles = lf::ceil_div(g.n_items, g.rows_per_tile);
+            g.rows = d_zero_rows;
+            groups.push_back(g);
+        }
+        L.n_groups = (int)groups.size() - L.group_begin;
+        if (L.n_groups > kMaxGroups)
+            return bail(lf::fail(LF_ERR_UNSUPPORTED, "partition %d needs %d tile groups (max %d)", p, L.n_groups, kMaxGroups));
+        for (int gi = L.group_begin; gi < (int)groups.size(); ++gi) L.tiles += groups[gi].n_tiles;
+        total_tiles += L.tiles;
+    }
+    if (!groups.empty()) {
+        LF_TRY(dev_alloc(plan, &plan->d_groups, groups.size()));
+        LF_TRY_HIP(hipMemcpy(plan->d_groups, groups.data(), groups.size() * sizeof(Group), hipMemcpyHostToDevice));
+    }
+
+    // persistent grid: enough workgroups to fill every CU at the kernel's occupancy
+    KernelSet ks;
+    LF_TRY(select_kernels(lpr, ch, b_dtype, &ks));
+    int occ = 0;
+    LF_TRY_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, ks.tiles, kWG, 0));
+    if (occ < 1) occ = 1;
+    plan->grid = std::max(kXcds, plan->num_cus * occ / kXcds * kXcds);
+
+    plan->info[0] = total_tiles;
+    plan->info[1] = plan->grid;
+    plan->info[2] = num_parts;
+    plan->info[3] = (int64_t)(sizeof(int2) * (kTileSlots + kTileRows) + sizeof(Group) * kMaxGroups);
+    plan->info[4] = (int64_t)heavy_rows.size();
+    plan->info[5] = n_partials;
+    plan->info[6] = n_zero;
+    plan->info[7] = occ;
+    *out_plan = plan;
+    return LF_OK;
+#undef LF_TRY
+#undef LF_TRY_HIP
+}
+
+int lf_spmm_info(const lf_spmm_plan* plan, int64_t* h_info) {
+    LF_REQUIRE(plan && h_info, LF_ERR_INVALID, "null argument");
+    std::memcpy(h_info, plan->info, sizeof(plan->info));
+    return LF_OK;
+}
+
+int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    LF_REQUIRE(plan, LF_ERR_INVALID, "plan is null");
+    if (plan->num_rows == 0) return LF_OK;
+    LF_REQUIRE(d_B && d_C, LF_ERR_INVALID, "B or C is null");
+    LF_REQUIRE((uintptr_t)d_B % 16 == 0 && (uintptr_t)d_C % 16 == 0, LF_ERR_INVALID, "B and C must be 16-byte aligned");
+    KernelSet ks;
+    if (int rc = select_kernels(plan->lpr, plan->ch, plan->b_dtype, &ks)) return rc;
+    for (int p = 0; p < plan->num_parts; ++p) {
+        const lf_spmm_plan::Launch& L = plan->launches[p];
+        if (L.n_groups == 0) continue;
+        LaunchArgs a{};
+        a.groups = plan->d_groups + L.group_begin;
+        a.n_groups = L.n_groups;
+        a.accumulate = p > 0 ? 1 : 0;
+        a.feat = plan->feat;
+        a.B = d_B;
+        a.C = d_C;
+        a.partials = plan->d_partials;
+        const long long want = (L.tiles + kXcds - 1) / kXcds * kXcds;
+        const int grid = (int)std::min<long long>(plan->grid, std::max<long long>(want, kXcds));
+        ks.tiles<<<grid, kWG, 0, s>>>(a);
+        LF_HIP(hipGetLastError());
+        if (L.n_heavy > 0) {
+            const int sw = kWG / plan->lpr;
+            const int fgrid = std::min((L.n_heavy + sw - 1) / sw, 1024);
+            ks.finalize<<<fgrid, kWG, 0, s>>>(plan->d_heavy + L.heavy_begin, L.n_heavy, a);
+            LF_HIP(hipGetLastError());
+        }
+    }
+    return LF_OK;
+}
+
+int lf_csr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values,
+                int64_t num_rows, int64_t num_cols, int32_t feat_size, int32_t b_dtype,
+                const void* d_B, float* d_C, lf_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    LF_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31) && num_cols >= 1, LF_ERR_INVALID, "bad shape");
+    if (num_rows == 0) return LF_OK;
+    LF_REQUIRE(d_indptr && d_B && d_C, LF_ERR_INVALID, "null argument");
+    LF_REQUIRE(b_dtype == LF_DTYPE_F32 || b_dtype == LF_DTYPE_BF16, LF_ERR_INVALID, "unknown B dtype %d", b_dtype);
+    LF_REQUIRE((uintptr_t)d_B % 16 == 0 && (uintptr_t)d_C % 16 == 0, LF_ERR_INVALID, "B and C must be 16-byte aligned");
+    int lpr, ch;
+    if (int rc = feature_shape(feat_size, b_dtype, &lpr, &ch)) return rc;
+    KernelSet ks;
+    if (int rc = select_kernels(lpr, ch, b_dtype, &ks)) return rc;
+    LaunchArgs a{};
+    a.feat = feat_size;
+    a.B = d_B;
+    a.C = d_C;
+    const int sw = kWG / lpr;
+    const int grid = (int)std::min<long long>((num_rows + sw - 1) / sw, 1 << 20);
+    ks.csr<<<grid, kWG, 0, s>>>(d_indptr, d_indices, d_values, num_rows, a);
+    LF_HIP(hipGetLastError());
+    return LF_OK;
+}
+
+int lf_spmm_time_ms(lf_spmm_plan* plan, const void* d_B, float* d_C, int32_t warmup, int32_t repeat,
+                    void* d_flush, size_t flush_bytes, float* h_ms, lf_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    LF_REQUIRE(plan && h_ms, LF_ERR_INVALID, "null argument");
+    LF_REQUIRE(warmup >= 0 && repeat >= 1, LF_ERR_INVALID, "bad warmup/repeat");
+    for (int i = 0; i < warmup; ++i)
+        if (int rc = lf_spmm_run(plan, d_B, d_C, stream)) return rc;
+    hipEvent_t t0, t1;
+    LF_HIP(hipEventCreate(&t0));
+    LF_HIP(hipEventCreate(&t1));
+    int rc = LF_OK;
+    for (int i = 0; i < repeat && rc == LF_OK; ++i) {
+        if (d_flush && flush_bytes >= 4) {
+            const long long words = (long long)(flush_bytes / 4);
+            fill_bytes_kernel<<<(int)std::min<long long>((words + 255) / 256, 8192), 256, 0, s>>>((uint32_t*)d_flush, words, (uint32_t)i);
+        }
+        hipError_t e = hipEventRecord(t0, s);
+        if (e == hipSuccess) {
+            rc = lf_spmm_run(plan, d_B, d_C, stream);
+            if (rc != LF_OK) break;
+            e = hipEventRecord(t1, s);
+        }
+        if (e == hipSuccess) e = hipEventSynchronize(t1);
+        if (e == hipSuccess) e = hipEventElapsedTime(&h_ms[i], t0, t1);
+        if (e != hipSuccess) rc = lf::fail(LF_ERR_HIP, "timing failed: %s", hipGetErrorString(e));
+    }
+    hipEventDestroy(t0);
+    hipEventDestroy(t1);
+    return rc;
+}
+
+}  // extern "C"

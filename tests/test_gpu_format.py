@@ -1,0 +1,133 @@
+"""GPU parity of the format pass (statistics, search, hyb composition) with the oracle.
+
+Everything goes through the C ABI (ctypes) behind the reference-shaped Python functions.
+Format structures must match bit for bit."""
+import numpy as np
+import pytest
+
+from oracle import liteform_oracle as O
+
+from helpers import assert_hyb_equal, mtx_from_rows, skewed_matrix, stats_from_oracle
+
+pytestmark = pytest.mark.gpu
+
+HAND = [[0, 1, 2, 5], [1], [], [0, 1, 2, 3, 4, 6], [2, 7], [0, 3, 4, 5, 6]]
+
+
+@pytest.fixture(scope="module")
+def fa():
+    from liteform_ae_amd import format_algos
+    return format_algos
+
+
+def test_hand_example_end_to_end(fa):
+    g = mtx_from_rows(HAND, (6, 8))
+    cfg = fa.search_bucket_config(g, 2, fa.CostModelSettings(32, 2))
+    assert cfg == [[1, 4], [1, 2]]
+    rows, cols, mask = fa.build_hyb_format(g, cfg)
+    assert rows[0][1].tolist() == [0, 3, 5]
+    assert cols[0][1].tolist() == [[0, 1, 2, 0], [0, 1, 2, 3], [0, 3, 0, 0]]
+    assert mask[0][1].tolist() == [[1, 1, 1, 0], [1, 1, 1, 1], [1, 1, 0, 0]]
+    assert rows[1][1].tolist() == [3, 5, 5]
+    assert cols[1][1].tolist() == [[4, 6], [4, 5], [6, 0]]
+    assert mask[1][1].tolist() == [[1, 1], [1, 1], [1, 0]]
+    assert rows[0][0].dtype == np.int64 and cols[0][1].shape == (3, 4)
+    assert_hyb_equal((rows, cols, mask), O.build_hyb_format_sequential(g, cfg))
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_bucket_stats_match_oracle(fa, seed):
+    rng = np.random.default_rng(40 + seed)
+    nr, nc = int(rng.integers(100, 3000)), int(rng.integers(100, 3000))
+    parts = int(rng.choice([1, 2, 3, 7, 16]))
+    g = skewed_matrix(rng, nr, nc, mean_deg=float(rng.choice([3, 8, 20])), heavy_rows=3, values=False)
+    stats, hist = fa.bucket_statistics(g, parts)
+    wstats, whist = stats_from_oracle(g, parts)
+    np.testing.assert_array_equal(stats, wstats)
+    np.testing.assert_array_equal(hist, whist)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_search_matches_oracle(fa, seed):
+    rng = np.random.default_rng(60 + seed)
+    nr, nc = int(rng.integers(200, 2500)), int(rng.integers(200, 2500))
+    parts = int(rng.choice([1, 2, 4, 8]))
+    feat = int(rng.choice([32, 128, 512]))
+    g = skewed_matrix(rng, nr, nc, mean_deg=8, heavy_rows=2, values=False)
+    try:
+        want = O.search_bucket_config(g, parts, O.OracleCostModelSettings(feat, parts))
+    except ValueError:
+        with pytest.raises(ValueError):
+            fa.search_bucket_config(g, parts, fa.CostModelSettings(feat, parts))
+        return
+    assert fa.search_bucket_config(g, parts, fa.CostModelSettings(feat, parts)) == want
+
+
+def test_single_nonzero_partition_raises_value_error(fa):
+    g = mtx_from_rows([[3]], (1, 8))
+    with pytest.raises(ValueError, match="only having 1 non-zero element"):
+        fa.search_bucket_config(g, 1, fa.CostModelSettings(32, 1))
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_builder_matches_sequential_oracle(fa, seed):
+    rng = np.random.default_rng(80 + seed)
+    nr, nc = int(rng.integers(30, 700)), int(rng.integers(30, 700))
+    parts = int(rng.choice([1, 2, 3, 5]))
+    g = skewed_matrix(rng, nr, nc, mean_deg=6, heavy_rows=2, values=False)
+    all_w = [1 << i for i in range(8)]
+    widths = [sorted(rng.choice(all_w, size=int(rng.integers(1, 6)), replace=False).tolist())
+              for _ in range(parts)]
+    got = fa.build_hyb_format(g, widths)
+    assert_hyb_equal(got, O.build_hyb_format_sequential(g, widths))
+
+
+def test_builder_with_searched_config_mid_size(fa):
+    rng = np.random.default_rng(7)
+    g = skewed_matrix(rng, 20000, 20000, mean_deg=12, heavy_rows=5, heavy_len=6000, values=False)
+    for parts in (1, 4):
+        cfg = fa.search_bucket_config(g, parts, fa.CostModelSettings(128, parts))
+        assert cfg == O.search_bucket_config(g, parts, O.OracleCostModelSettings(128, parts))
+        assert_hyb_equal(fa.build_hyb_format(g, cfg), O.build_hyb_format_closed_form(g, cfg))
+
+
+def test_builder_edge_cases(fa):
+    # empty matrix rows, an empty partition, a single bucket of width 1 holding a long row
+    g = mtx_from_rows([[], [0, 1, 2, 3, 4], [], [1]], (4, 16))
+    for widths in ([[1], []], [[8], []], [[1, 2, 4, 8], []]):
+        assert_hyb_equal(fa.build_hyb_format(g, widths), O.build_hyb_format_sequential(g, widths))
+    with pytest.raises(IndexError):
+        fa.build_hyb_format(g, [[], [4]])                 # nonzeros in a partition without widths
+    with pytest.raises(AssertionError):
+        fa.build_hyb_format(g, [[3], []])                 # not a power of two
+    # empty buckets are kept with shapes (0,), (0, W)   (format_algos.py:365-368)
+    rows, cols, mask = fa.build_hyb_format(g, [[1, 2, 4, 8], []])
+    assert rows[0][1].shape == (0,) and cols[0][1].shape == (0, 2) and mask[0][2].shape == (0, 4)
+
+
+def test_duplicate_coo_entries(fa):
+    """COO duplicates raise the degree but not the fill (format_algos.py:250-254)."""
+    from liteform_ae_amd.format_matrix_market import MTX
+    rng = np.random.default_rng(11)
+    r = rng.integers(0, 50, size=600)
+    c = rng.integers(0, 64, size=600)
+    g = MTX.from_coo(r, c, (50, 64))
+    assert g.num_edges() != g.adj_tensors("csr")[1].shape[0]      # there are duplicates
+    for parts in (1, 2):
+        widths = [[2, 8, 16]] * parts
+        assert_hyb_equal(fa.build_hyb_format(g, widths), O.build_hyb_format_sequential(g, widths))
+        stats, hist = fa.bucket_statistics(g, parts)
+        wstats, whist = stats_from_oracle(g, parts)
+        np.testing.assert_array_equal(stats, wstats)
+        np.testing.assert_array_equal(hist, whist)
+
+
+def test_workload_shapes_scaled(fa):
+    from liteform_ae_amd.synthetic import make_workload
+    for name, scale, parts in (("cfg1", 1.0, 1), ("cfg2", 0.05, 2), ("cfg3", 0.005, 1), ("cfg3", 0.005, 4),
+                               ("cfg4", 0.004, 1), ("cfg5", 0.01, 2)):
+        wl = make_workload(name, scale)
+        g = wl.matrix
+        cfg = fa.search_bucket_config(g, parts, fa.CostModelSettings(wl.feat_size, parts))
+        assert cfg == O.search_bucket_config(g, parts, O.OracleCostModelSettings(wl.feat_size, parts)), name
+        assert_hyb_equal(fa.build_hyb_format(g, cfg), O.build_hyb_format_closed_form(g, cfg))
