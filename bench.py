@@ -96,6 +96,8 @@ def main():
     ap.add_argument("--cost-model", default="reference", choices=["reference", "gfx950"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB device copy, so a counter run reads a known size")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -166,6 +168,14 @@ def main():
     ev_cold_ms = plan.time_ms(B_dev, C_dev, warmup=0, repeat=max(3, args.steps // 3), flush=flush)
     del flush
     kernel_ms = float(np.mean(ev_ms))
+
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")      # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     flops = 2.0 * nnz * feat
     algo = algorithmic_bytes(nnz, rows, cols, feat, b_bytes)
