@@ -91,9 +91,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg3")
     ap.add_argument("--feat", type=int, default=0, help="dense columns N (default: the workload's)")
-    ap.add_argument("--parts", type=int, default=0, help="column partitions (default: the workload's, or 1)")
+    ap.add_argument("--parts", type=int, default=0,
+                    help="column partitions (default: the workload's; measured choice where it names none)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the matrix (testing only)")
-    ap.add_argument("--cost-model", default="reference", choices=["reference", "gfx950"])
+    ap.add_argument("--cost-model", default="gfx950", choices=["reference", "gfx950"],
+                    help="cost function of the bucket-width search (the reference's, or the MI355X one)")
+    ap.add_argument("--widths", default="", help="bucket widths instead of the searched ones, "
+                    "e.g. '1,2,4,8;1,2,4' (partitions separated by ';')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--copy-calibration", action="store_true",
@@ -117,12 +121,12 @@ def main():
     t0 = time.perf_counter()
     wl = make_workload(args.workload, args.scale)
     feat = args.feat or wl.feat_size
-    parts = args.parts or wl.num_parts or 1
+    parts = args.parts or wl.num_parts
     g = wl.matrix
     rows, cols = wl.shape
     nnz = wl.nnz
     t_gen = time.perf_counter() - t0
-    print(f"[bench] {wl.name}: {rows} x {cols}, nnz {nnz}, N {feat}, P {parts}, B {wl.b_dtype} "
+    print(f"[bench] {wl.name}: {rows} x {cols}, nnz {nnz}, N {feat}, P {parts or 'auto'}, B {wl.b_dtype} "
           f"(generated in {t_gen:.1f} s)", file=sys.stderr, flush=True)
 
     B_host = make_dense(cols, feat, wl.seed)
@@ -138,11 +142,22 @@ def main():
     # ---- format composition (GPU): search = what the reference times as time_bucket
     fa._device_csr(g)                       # upload CSR once, outside the timed parts
     torch.cuda.synchronize()
+    part_timings = None
+    if not parts:                           # the workload leaves the partition count open
+        t0 = time.perf_counter()
+        parts, part_timings = fa.choose_num_partitions(g, feat, wl.b_dtype, cost_model=args.cost_model,
+                                                       return_timings=True)
+        print(f"[bench] partition count chosen by measurement: {parts} from {part_timings} "
+              f"({time.perf_counter() - t0:.2f} s)", file=sys.stderr, flush=True)
     cfg_obj = fa.CostModelSettings(feat, parts, cost_model=args.cost_model)
     fa.search_bucket_config(g, parts, cfg_obj)            # warm
     t0 = time.perf_counter()
     config = fa.search_bucket_config(g, parts, cfg_obj)
     search_ms = (time.perf_counter() - t0) * 1e3
+    if args.widths:
+        config = [[int(w) for w in part.split(",") if w] for part in args.widths.split(";")]
+        if len(config) == 1 and parts > 1:
+            config = config * parts
     fa.build_hyb_format_device(g, config)                 # warm
     t0 = time.perf_counter()
     fmt = fa.build_hyb_format_device(g, config)
@@ -200,6 +215,7 @@ def main():
             "workload": f"{wl.name}: {wl.description}" + ("" if args.scale == 1.0 else f" (scale {args.scale})"),
             "rows": rows, "cols": cols, "nnz": nnz, "feat_size": feat, "num_parts": parts,
             "bucket_widths": config, "cost_model": args.cost_model,
+            "num_parts_candidates_ms": part_timings,
         },
         "roofline": {
             "bound": "hbm",

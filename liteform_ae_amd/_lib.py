@@ -26,7 +26,9 @@ LF_DTYPE_BF16 = 1
 LF_COST_REFERENCE = 0
 LF_COST_GFX950 = 1
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "liblfhip.so")
+# LITEFORM_HIP_LIB points at another build of the same library (kernel tuning experiments)
+LIB_PATH = os.environ.get("LITEFORM_HIP_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)),
+                                                              "liblfhip.so")
 
 i32p = C.POINTER(C.c_int32)
 i64p = C.POINTER(C.c_int64)

@@ -34,21 +34,23 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin)")
 
 
-def build(verbose: bool = True) -> str:
+def build(verbose: bool = True, extra_flags=(), out: str = LIB, objdir: str | None = None) -> str:
+    """Compile every source and link `out`.  `extra_flags` (e.g. "-DLF_UNROLL=16") are for
+    kernel-tuning builds loaded through the LITEFORM_HIP_LIB environment variable."""
     hipcc = hipcc_path()
-    objdir = os.path.join(HERE, "build")
+    objdir = objdir or os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     objs = []
     for src in SOURCES:
         obj = os.path.join(objdir, os.path.splitext(src)[0] + ".o")
-        cmd = [hipcc, *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC]
+        cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-I", os.path.join(ROOT, "include"), "-I", CSRC]
         if src.endswith(".cpp"):
             cmd += ["-x", "hip"]
         cmd += ["-c", os.path.join(CSRC, src), "-o", obj]
         _run(cmd, verbose)
         objs.append(obj)
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], verbose)
-    return LIB
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *objs], verbose)
+    return out
 
 
 def _run(cmd, verbose):

@@ -104,25 +104,28 @@ double reference_cost(const Pool& pool, const int64_t* hist, int nmask, int32_t 
     return cost;
 }
 
-// Traffic model for the gfx950 kernels, in bytes.  The B gather (nnz * feat * 4) and the C
-// store are the same for every state of the fold chain, so only what a fold changes is
-// priced: slab bytes (8 per slot, padding included), per-ELL-row bytes (row id + meta), and
-// the cost of splitting a source row over several ELL rows, whose partial sums are combined
-// through LDS or, beyond a few thousand slots, through a partial-row buffer in HBM.
+// Cost of a state for the gfx950 kernels, in bytes of HBM-traffic equivalent.  The B gather
+// (nnz * feat * sizeof(B)) and the C store are the same for every state of the fold chain, so
+// only what a fold changes is priced:
+//   * 8 bytes per slab slot (column + value are streamed once, padding included);
+//   * kRowBytes per ELL row: 8 bytes of row id + meta, and the fixed work of starting a row
+//     (descriptor reads, loop set-up, a sub-wave slot left idle on continuation rows).
+// kRowBytes was fitted on MI355X: on the 2.45M-row power-law graph at N = 128 every extra
+// million ELL rows costs 0.07-0.2 ms at ~6 TB/s, i.e. 400-1200 bytes each, while padded slots
+// cost no more than their slab bytes because a padded slot re-reads a row that is already
+// in flight.  With these weights a fold pays only when it removes far more padding than it
+// adds rows, which on the benchmark workloads keeps the initial power-of-two widths.
+constexpr double kSlotBytes = 8.0;
+constexpr double kRowBytes = 600.0;
+
 double gfx950_cost(const Pool& pool, const int64_t* hist, int nmask, int32_t feat, int32_t parts) {
     (void)hist;
     (void)nmask;
-    const int32_t max_w = pool.max_width();
+    (void)feat;
+    (void)parts;
     double cost = 0.0;
-    for (const Bucket& b : pool.items) {
-        const double slots = (double)b.num_rows * (double)b.width;
-        cost += 8.0 * slots + 8.0 * (double)b.num_rows;
-        if (b.width == max_w) {
-            const double extra = (double)std::max<int64_t>(0, b.num_rows - b.out_rows);
-            cost += extra * (double)feat * 4.0 * 0.25;
-        }
-        cost += (double)b.out_rows * (double)feat * 4.0 * (parts > 1 ? 2.0 : 1.0);
-    }
+    for (const Bucket& b : pool.items)
+        cost += kSlotBytes * (double)b.num_rows * (double)b.width + kRowBytes * (double)b.num_rows;
     return cost;
 }
 

@@ -27,6 +27,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -35,13 +36,19 @@
 namespace {
 
 constexpr int kWG = 256;            // threads per workgroup (4 wavefronts)
-constexpr int kTileSlots = 2048;    // (col, val) pairs staged in LDS per tile: 16 KiB
-constexpr int kTileRows = 512;      // ELL rows per tile at most
+#ifndef LF_TILE_SLOTS
+#define LF_TILE_SLOTS 1024
+#endif
+#ifndef LF_UNROLL
+#define LF_UNROLL 8
+#endif
+constexpr int kTileSlots = LF_TILE_SLOTS;   // (col, val) pairs staged in LDS per tile: 8 KiB
+constexpr int kTileRows = 512;      // ELL rows per tile at most (<= kTileSlots)
 constexpr int kHeavySlots = 1024;   // a source row with more slab slots is split into chunks
 constexpr int kChunkSlots = 2048;   // slots per chunk (a whole number of ELL rows)
 constexpr int kXcds = 8;
 constexpr int kMaxGroups = 48;      // tile groups per launch
-constexpr int kUnroll = 8;          // B-row gathers in flight per sub-wave
+constexpr int kUnroll = LF_UNROLL;  // B-row gathers in flight per sub-wave
 constexpr uint32_t kMetaLenMask = 0x7FFu;
 constexpr int kMetaLenBits = 11;
 
@@ -137,19 +144,19 @@ template <int LPR, int CH, int VEC> struct Lane {
     }
 };
 
-template <int LPR, int CH, typename BT>
+template <int U, int LPR, int CH, typename BT>
 __device__ __forceinline__ void gather_fma(const void* B, const Lane<LPR, CH, Dense<BT>::kVec>& ln,
-                                           const int (&col)[kUnroll], const float (&val)[kUnroll],
+                                           const int (&col)[U], const float (&val)[U],
                                            Acc<CH, Dense<BT>::kVec>& acc) {
     constexpr int VEC = Dense<BT>::kVec;
-    float x[kUnroll][CH][VEC];
+    float x[U][CH][VEC];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int c = 0; c < CH; ++c)
             Dense<BT>::load(B, (size_t)(uint32_t)col[u] * (size_t)ln.feat + ln.f[c], x[u][c]);
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int c = 0; c < CH; ++c)
 #pragma unroll
@@ -183,6 +190,7 @@ __device__ __forceinline__ void stream_slots(const int32_t* __restrict__ cols, c
                                              long long base, int total, const void* B,
                                              const Lane<LPR, CH, Dense<BT>::kVec>& ln,
                                              Acc<CH, Dense<BT>::kVec>& acc) {
+    constexpr int U = kUnroll < LPR ? kUnroll : LPR;
     if (total <= 0) return;
     const int c_first = cols[base];
     for (int off = 0; off < total; off += LPR) {
@@ -191,22 +199,22 @@ __device__ __forceinline__ void stream_slots(const int32_t* __restrict__ cols, c
         const int my_c = have ? cols[base + idx] : c_first;
         const float my_v = have ? (vals ? vals[base + idx] : 1.f) : 0.f;
         const int cnt = min(LPR, total - off);
-        for (int j = 0; j < cnt; j += kUnroll) {
-            int c[kUnroll];
-            float v[kUnroll];
+        for (int j = 0; j < cnt; j += U) {
+            int c[U];
+            float v[U];
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
+            for (int u = 0; u < U; ++u) {
                 c[u] = __shfl(my_c, j + u, LPR);
                 v[u] = __shfl(my_v, j + u, LPR);
             }
-            gather_fma<LPR, CH, BT>(B, ln, c, v, acc);
+            gather_fma<U, LPR, CH, BT>(B, ln, c, v, acc);
         }
     }
 }
 
 // ------------------------------------------------------------------------------------
-// Tile bodies.  `smem` is the workgroup's LDS: kTileSlots int2 pairs followed by
-// kTileRows int2 (row, meta) entries.
+// Tile bodies.  s_pairs / s_rm point into the workgroup's LDS: kTileSlots (col, val) pairs
+// followed by kTileRows (row, meta) entries.
 
 // Narrow bucket: W slots per ELL row, rows independent (one ELL row per source row).
 // RPI rows are processed together by a sub-wave so that kUnroll gathers are in flight
@@ -256,7 +264,7 @@ __device__ __forceinline__ void ell_tile_narrow(const int2* s_pairs, const int2*
     }
 }
 
-// Bucket with W >= kUnroll staged in LDS: one ELL row per sub-wave at a time.
+// Bucket with W >= kUnroll (a multiple of it) staged in LDS: one ELL row per sub-wave at a time.
 template <int LPR, int CH, typename BT>
 __device__ __forceinline__ void ell_tile_wide(const int2* s_pairs, const int2* s_rm, int n, int log_w,
                                               const LaunchArgs& a, int sw, int sl) {
@@ -279,7 +287,7 @@ __device__ __forceinline__ void ell_tile_wide(const int2* s_pairs, const int2* s
                 c[u] = j + u < len ? cv.x : c0;
                 v[u] = __int_as_float(cv.y);
             }
-            gather_fma<LPR, CH, BT>(a.B, ln, c, v, acc);
+            gather_fma<kUnroll, LPR, CH, BT>(a.B, ln, c, v, acc);
         }
         store_row<LPR, CH, VEC>(a.C, rm.x, ln, acc, a.accumulate);
     }
@@ -314,6 +322,10 @@ __device__ __forceinline__ void run_ell_tile(const Group& g, long long tile, int
         case 0: ell_tile_narrow<1, LPR, CH, BT>(s_pairs, s_rm, n, a, sw, sl); break;
         case 1: ell_tile_narrow<2, LPR, CH, BT>(s_pairs, s_rm, n, a, sw, sl); break;
         case 2: ell_tile_narrow<4, LPR, CH, BT>(s_pairs, s_rm, n, a, sw, sl); break;
+        case 3:
+            if constexpr (kUnroll > 8) ell_tile_narrow<8, LPR, CH, BT>(s_pairs, s_rm, n, a, sw, sl);
+            else ell_tile_wide<LPR, CH, BT>(s_pairs, s_rm, n, g.log_w, a, sw, sl);
+            break;
         default: ell_tile_wide<LPR, CH, BT>(s_pairs, s_rm, n, g.log_w, a, sw, sl); break;
     }
 }
@@ -406,8 +418,13 @@ __device__ __forceinline__ void run_chunk_tile(const Group& g, long long tile, f
 template <int LPR, int CH, typename BT>
 __global__ void __launch_bounds__(kWG)
 spmm_partition_kernel(LaunchArgs a) {
-    __shared__ int2 s_pairs[kTileSlots];
-    __shared__ int2 s_rm[kTileRows];
+    // one LDS buffer, used either as the staged tile ((col, val) pairs then (row, meta)
+    // entries) or as the reduction scratch of a chunk tile (one accumulator per thread)
+    constexpr int kStageBytes = (kTileSlots + kTileRows) * (int)sizeof(int2);
+    constexpr int kReduceBytes = kWG * CH * Dense<BT>::kVec * (int)sizeof(float);
+    __shared__ __align__(16) char s_raw[kStageBytes > kReduceBytes ? kStageBytes : kReduceBytes];
+    int2* s_pairs = reinterpret_cast<int2*>(s_raw);
+    int2* s_rm = s_pairs + kTileSlots;
     __shared__ Group s_groups[kMaxGroups];
 
     {   // the group table is small: copy it into LDS once
@@ -437,7 +454,7 @@ spmm_partition_kernel(LaunchArgs a) {
                 case kEll: run_ell_tile<LPR, CH, BT>(g, tile, s_pairs, s_rm, a); break;
                 case kSeg: run_seg_tile<LPR, CH, BT>(g, tile, a); break;
                 case kZero: run_zero_tile<LPR, CH, BT>(g, tile, a); break;
-                default: run_chunk_tile<LPR, CH, BT>(g, tile, reinterpret_cast<float*>(s_pairs), a); break;
+                default: run_chunk_tile<LPR, CH, BT>(g, tile, reinterpret_cast<float*>(s_raw), a); break;
             }
             v += per_xcd;
         }
@@ -909,12 +926,17 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     int occ = 0;
     LF_TRY_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, ks.tiles, kWG, 0));
     if (occ < 1) occ = 1;
+    if (const char* e = getenv("LF_SPMM_WGS_PER_CU")) occ = std::max(1, atoi(e));
     plan->grid = std::max(kXcds, plan->num_cus * occ / kXcds * kXcds);
 
     plan->info[0] = total_tiles;
     plan->info[1] = plan->grid;
     plan->info[2] = num_parts;
-    plan->info[3] = (int64_t)(sizeof(int2) * (kTileSlots + kTileRows) + sizeof(Group) * kMaxGroups);
+    {
+        hipFuncAttributes fa;
+        LF_TRY_HIP(hipFuncGetAttributes(&fa, reinterpret_cast<const void*>(ks.tiles)));
+        plan->info[3] = (int64_t)fa.sharedSizeBytes;
+    }
     plan->info[4] = (int64_t)heavy_rows.size();
     plan->info[5] = n_partials;
     plan->info[6] = n_zero;

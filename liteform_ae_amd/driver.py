@@ -1,0 +1,126 @@
+"""End-to-end flow of the reference's driver for matrices that use the CELL (hyb) format.
+
+Mirrors the CELL branch of ``playground_pipline/proc05.spmm.end-to-end.py:127-190`` and its
+result table (proc05.spmm.end-to-end.py:273-286): for every matrix and every feature size
+the column-partition count is chosen, the bucket-width search is timed (``time_bucket(s)``),
+the hyb format is composed and the fused kernel is timed (``time_exe_our(ms)``).
+
+Differences: the reference predicts the format (CELL or BCSR) and the partition count with
+RandomForest models; the partition model is not distributed and the BSR path is outside
+this library, so every matrix is run as CELL and the partition count is measured
+(``choose_num_partitions``) or given.  Extra columns report GFLOP/s and compose time.
+
+    python -m liteform_ae_amd.driver --synthetic cfg2 --feat 32 64 128
+    python -m liteform_ae_amd.driver --dataset path/to/matrix.mtx
+"""
+from __future__ import annotations
+
+import argparse
+import math
+import sys
+import time
+
+import numpy as np
+
+from .format_matrix_market import MTX
+
+FEAT_SIZES = (32, 64, 128, 256, 512)        # proc05.spmm.end-to-end.py:141
+
+
+def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="reference",
+                   check_correctness=False, out_csv=None, keep_values=False):
+    """Runs the flow for an iterable of MTX objects and returns a pandas DataFrame with the
+    reference's columns.  ``num_parts``: None = measure per (matrix, feature size); an int;
+    or a callable ``(g, feat_size) -> int``."""
+    import pandas as pd
+    import torch
+
+    from . import format_algos as fa
+
+    table = {k: [] for k in ("name", "format", "feat_size", "num_parts", "time_select(s)",
+                             "time_num_parts(s)", "time_bucket(s)", "time_exe_our(ms)",
+                             "time_compose(ms)", "GFLOP/s", "bucket_config")}
+    for g in matrices:
+        print(f"\nGo to name {g.name} ...")
+        fmt_name, time_select = "CELL", 0.0
+        for feat in feat_sizes:
+            t0 = time.perf_counter()
+            if num_parts is None:
+                parts = fa.choose_num_partitions(g, feat, cost_model=cost_model)
+            elif callable(num_parts):
+                parts = int(num_parts(g, feat))
+            else:
+                parts = int(num_parts)
+            time_parts = time.perf_counter() - t0
+            print(f"name: {g.name} num_parts: {parts} time(s): {time_parts}")
+
+            print("Configuring ...", flush=True)
+            t0 = time.perf_counter()                                   # proc05:153-157
+            cfg = fa.CostModelSettings(feat_size=feat, num_parts=parts, cost_model=cost_model)
+            bucket_config = fa.search_bucket_config(g, parts, cfg)
+            time_bucket = time.perf_counter() - t0
+
+            x = torch.ones((g.num_dst_nodes(), feat))                  # proc05:162
+            y_ndarray = g.dot(x.numpy()) if check_correctness else None
+            compose_ms = float("nan")
+            try:
+                if keep_values:
+                    hyb = fa.build_hyb_format_device(g, bucket_config)
+                else:
+                    hyb = fa.build_hyb_format_device(g, bucket_config, with_values=False)
+                compose_ms = hyb.compose_ms
+                exe_time = fa.bench_hyb_with_config(g, x, y_ndarray, feat_size=feat, bucket_widths=bucket_config,
+                                                    bucketing_format=hyb, coarsening_factor=2,
+                                                    num_col_parts=parts, use_implicit_unroll=True,
+                                                    check_correctness=check_correctness)
+                print(f"name: {g.name} format: {fmt_name} feat_size: {feat} num_partitions: {parts} "
+                      f"cost_model_config: {cfg} bucket_config: {bucket_config} exe_time: {exe_time}", flush=True)
+            except Exception as e:                                     # proc05:178-180
+                exe_time = math.inf
+                print(e, file=sys.stderr)
+            table["name"].append(g.name)
+            table["format"].append(fmt_name)
+            table["feat_size"].append(feat)
+            table["num_parts"].append(parts)
+            table["time_select(s)"].append(time_select)
+            table["time_num_parts(s)"].append(time_parts)
+            table["time_bucket(s)"].append(time_bucket)
+            table["time_exe_our(ms)"].append(exe_time)
+            table["time_compose(ms)"].append(compose_ms)
+            table["GFLOP/s"].append(2.0 * g.num_edges() * feat / (exe_time * 1e-3) / 1e9 if exe_time > 0 else 0.0)
+            table["bucket_config"].append(str(bucket_config))
+    df = pd.DataFrame(data=table)
+    print(df.to_string())
+    if out_csv:
+        df.to_csv(out_csv, index=False)
+    return df
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser("CELL-format SpMM end to end")
+    ap.add_argument("--dataset", "-d", nargs="*", default=[], help="MatrixMarket (.mtx) files")
+    ap.add_argument("--synthetic", nargs="*", default=[], help="synthetic workloads: cfg1 .. cfg5")
+    ap.add_argument("--scale", type=float, default=1.0)
+    ap.add_argument("--feat", type=int, nargs="*", default=list(FEAT_SIZES))
+    ap.add_argument("--num-parts", type=int, default=0, help="0 = choose by measurement")
+    ap.add_argument("--cost-model", default="reference", choices=["reference", "gfx950"])
+    ap.add_argument("--check", action="store_true", help="compare with scipy (rtol 1e-4) as the reference can")
+    ap.add_argument("--csv", default="", help="write the table to this file")
+    args = ap.parse_args(argv)
+    mats = [MTX(path) for path in args.dataset]
+    if args.synthetic:
+        from .synthetic import make_workload
+        for name in args.synthetic:
+            wl = make_workload(name, args.scale)
+            coo = wl.matrix.coo_mtx                             # the reference's matrices are unweighted
+            mats.append(MTX.from_coo(coo.row, coo.col, coo.shape, name=wl.matrix.name))
+    if not mats:
+        ap.print_help(sys.stderr)
+        return 2
+    run_end_to_end(mats, feat_sizes=args.feat, num_parts=args.num_parts or None, cost_model=args.cost_model,
+                   check_correctness=args.check, out_csv=args.csv or None)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

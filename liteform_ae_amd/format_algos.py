@@ -34,7 +34,8 @@ from .format_matrix_market import MTX, Bucket  # noqa: F401  (re-exported like t
 
 __all__ = ["build_hyb_format", "bench_hyb_with_config", "search_bucket_config",
            "CostModelSettings", "bench_naive",
-           "build_hyb_format_device", "HybFormat", "HybSpMM", "spmm_hyb", "spmm_csr"]
+           "build_hyb_format_device", "HybFormat", "HybSpMM", "spmm_hyb", "spmm_csr",
+           "guess_num_partitions", "choose_num_partitions"]
 
 WIDTH_LIMIT = 1024   # format_algos.py:821
 
@@ -496,3 +497,50 @@ def bench_naive(g, x, y_ndarray, feat_size=128, coarsening_factor=2, check_corre
     dur = float(np.mean([s.elapsed_time(e) for s, e in zip(starts, ends)]))
     print("csr naive time: {:.5f} ms".format(dur))
     return dur
+
+
+# --------------------------------------------------------------------------- partition count
+MALL_BYTES = 256 << 20        # MI355X memory-side cache (Infinity Cache)
+
+
+def guess_num_partitions(g, feat_size: int, b_dtype: str = "f32") -> int:
+    """Column-partition count without measuring.  The reference predicts it with a trained
+    RandomForest (proc05.spmm.end-to-end.py:82-97) whose model file is not distributed; this
+    rule states what measurements on MI355X showed instead: partitions pay only when B is
+    several times larger than the 256 MB memory-side cache *and* B rows are reused often
+    (nnz / cols), because every extra partition re-reads and re-writes C once and adds one
+    ELL row per (row, partition) segment."""
+    elem = 2 if b_dtype == "bf16" else 4
+    b_bytes = g.num_dst_nodes() * feat_size * elem
+    reuse = g.num_edges() / max(1, g.num_dst_nodes())
+    if b_bytes <= 0.75 * MALL_BYTES or reuse < 8:
+        return 1
+    return int(min(4, max(1, round(b_bytes / (2.5 * MALL_BYTES)))))
+
+
+def choose_num_partitions(g, feat_size: int, b_dtype: str = "f32", candidates: Sequence[int] = (1, 2, 3, 4),
+                          cost_model: str = "gfx950", runs: int = 3, return_timings: bool = False):
+    """Column-partition count by measurement: composes the format for every candidate and
+    times the fused kernel (a few runs each); returns the fastest.  Takes the place of the
+    reference's partition predictor (proc05.spmm.end-to-end.py:142)."""
+    torch = _torch()
+    want = torch.float32 if b_dtype == "f32" else torch.bfloat16
+    B = torch.zeros((g.num_dst_nodes(), feat_size), dtype=want, device="cuda")
+    Cout = torch.empty((g.num_src_nodes(), feat_size), dtype=torch.float32, device="cuda")
+    timings = {}
+    for p in candidates:
+        try:
+            cfg = search_bucket_config(g, p, CostModelSettings(feat_size, p, cost_model=cost_model))
+        except ValueError:
+            continue                      # a partition with a single nonzero: not a usable split
+        fmt = build_hyb_format_device(g, cfg)
+        plan = HybSpMM(fmt, feat_size, b_dtype)
+        try:
+            timings[p] = float(np.min(plan.time_ms(B, Cout, warmup=1, repeat=runs)))
+        finally:
+            plan.close()
+        del fmt
+    if not timings:
+        raise ValueError("no candidate partition count is usable for this matrix")
+    best = min(timings, key=timings.get)
+    return (best, timings) if return_timings else best

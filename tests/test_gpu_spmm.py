@@ -191,3 +191,20 @@ def test_workloads_scaled(fa, torch):
         wl = make_workload(name, scale)
         cfg = fa.search_bucket_config(wl.matrix, parts, fa.CostModelSettings(wl.feat_size, parts))
         check(fa, torch, wl.matrix, cfg, wl.feat_size, wl.b_dtype, seed=wl.seed)
+
+
+def test_partition_chooser_and_driver_table(fa, torch):
+    from liteform_ae_amd import driver
+    rng = np.random.default_rng(41)
+    g = skewed_matrix(rng, 3000, 3000, mean_deg=8, heavy_rows=2, values=False)
+    g.name = "toy"
+    best, timings = fa.choose_num_partitions(g, 64, candidates=(1, 2), return_timings=True)
+    assert best in timings and set(timings) == {1, 2}
+    assert fa.guess_num_partitions(g, 64) == 1            # B is far smaller than the memory-side cache
+    import os
+    os.environ["LF_REPEAT"] = "2"
+    os.environ["LF_WARMUP"] = "1"
+    df = driver.run_end_to_end([g], feat_sizes=(32, 64), num_parts=2, check_correctness=True)
+    assert list(df.columns[:8]) == ["name", "format", "feat_size", "num_parts", "time_select(s)",
+                                    "time_num_parts(s)", "time_bucket(s)", "time_exe_our(ms)"]
+    assert len(df) == 2 and (df["format"] == "CELL").all() and np.isfinite(df["time_exe_our(ms)"]).all()
