@@ -9,8 +9,10 @@ configuration the headline metric is quoted on.  Prints one JSON line:
 
   value            GFLOP/s = 2 * nnz * N / t, from the wall time of K back-to-back steps
   roofline         HBM: algorithmic bytes per step / average kernel time of a step measured
-                   with HIP events on the launch stream; traffic = L2<->fabric bytes per
-                   step from rocprofv3 counters when a measurement is on file
+                   with HIP events on the launch stream (a step is one launch per column
+                   partition; bytes and time are both summed over them, so the ratio is also
+                   the per-launch one); traffic = L2<->fabric bytes per step from rocprofv3
+                   counters when a measurement is on file
   format_compose   bucket-width search and slab build times (GPU), reported beside it
   cpu_baseline     scipy CSR @ dense (the reference's own CPU product, one thread) on a
                    bounded sample of rows of the same matrix
@@ -224,6 +226,7 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 5),
             "traffic": traffic,
+            "launches_per_step": parts,
             "kernel_ms": round(kernel_ms, 4),
             "kernel_ms_min": round(float(np.min(ev_ms)), 4),
             "kernel_ms_cold": round(float(np.mean(ev_cold_ms)), 4),
