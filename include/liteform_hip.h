@@ -74,6 +74,8 @@ const char* lf_status_string(int status);
  * d_seg_deg (optional, [num_parts][num_rows] int32) carries per-(partition,row) degrees
  * counted from raw COO triplets as the reference does (format_algos.py:846-849); when
  * NULL the degrees are the CSR segment lengths (identical for duplicate-free input).
+ * h_colhist may be NULL: the column sets are then not collected (LF_COST_GFX950 does not
+ * read them), which leaves one pass over indptr.
  * Synchronises the stream before returning (host outputs).
  * ------------------------------------------------------------------------------------ */
 size_t lf_stats_workspace_bytes(int64_t num_rows, int64_t num_cols, int32_t num_parts);

@@ -119,8 +119,10 @@ __device__ __forceinline__ void width_class(int deg, int kmax, int& k, int& cost
 
 // One thread per (row, partition) segment; blockIdx.y is the partition.
 //   stats[p][k] += {cost rows, nnz, 1}
-//   colmask[c]  |= 1 << k        for every column c of the segment
+//   colmask[c]  |= 1 << k        for every column c of the segment   (skipped when colmask is null)
 // Long segments are walked by the whole wave so that a heavy row does not serialise.
+// (One mask word per column measured faster than one bit plane per class: the planes fit
+// the L2 but 32 columns then share a word and the atomics collide.)
 __global__ void __launch_bounds__(kBlock)
 bucket_stats_kernel(SegView v, const int32_t* __restrict__ indices, const int32_t* __restrict__ seg_deg,
                     int kmax, uint32_t* __restrict__ colmask, unsigned long long* __restrict__ stats) {
@@ -144,6 +146,7 @@ bucket_stats_kernel(SegView v, const int32_t* __restrict__ indices, const int32_
         atomicAdd(&s_stats[k * LF_STATS_FIELDS + 1], (unsigned long long)deg);
         atomicAdd(&s_stats[k * LF_STATS_FIELDS + 2], 1ull);
     }
+    if (colmask == nullptr) bit = 0;
     const bool is_long = bit != 0 && fill > kLongSeg;
     if (bit != 0 && !is_long) {
         for (int i = 0; i < fill; ++i) {
@@ -517,7 +520,7 @@ int lf_bucket_stats(const int32_t* d_indptr, const int32_t* d_indices, const int
                     lf_stream_t stream) {
     hipStream_t s = (hipStream_t)stream;
     if (int rc = check_common(d_indptr, d_indices, num_rows, num_cols, num_parts)) return rc;
-    LF_REQUIRE(h_stats && h_colhist, LF_ERR_INVALID, "output pointers are null");
+    LF_REQUIRE(h_stats, LF_ERR_INVALID, "h_stats is null");
     LF_REQUIRE(lf::is_pow2(width_limit) && width_limit <= (1 << (LF_MAX_CLASSES - 1)), LF_ERR_INVALID,
                "width_limit must be a power of two <= %d", 1 << (LF_MAX_CLASSES - 1));
     const StatsLayout L = stats_layout(num_rows, num_cols, num_parts);
@@ -532,7 +535,10 @@ int lf_bucket_stats(const int32_t* d_indptr, const int32_t* d_indices, const int
     const size_t stats_bytes = (size_t)num_parts * LF_MAX_CLASSES * LF_STATS_FIELDS * 8;
     const size_t hist_bytes = (size_t)num_parts * (1 << LF_MAX_CLASSES) * 8;
 
-    LF_HIP(fill_u32(colmask, (L.total - L.colmask) / 4, 0u, s));   // colmask, stats and hist
+    if (h_colhist)
+        LF_HIP(fill_u32(colmask, (L.total - L.colmask) / 4, 0u, s));   // colmask, stats and hist
+    else
+        LF_HIP(fill_u32(stats, (L.total - L.stats) / 4, 0u, s));
     if (num_rows > 0) {
         const int nblk = (int)((num_rows + kBlock - 1) / kBlock);
         if (num_parts > 1) {
@@ -541,14 +547,17 @@ int lf_bucket_stats(const int32_t* d_indptr, const int32_t* d_indices, const int
         }
         SegView v{d_indptr, bnd, num_rows, num_parts};
         bucket_stats_kernel<<<dim3(nblk, num_parts), kBlock, 0, s>>>(v, d_indices, d_seg_deg,
-                                                                     lf::ilog2(width_limit), colmask, stats);
+                                                                     lf::ilog2(width_limit),
+                                                                     h_colhist ? colmask : nullptr, stats);
         LF_HIP(hipGetLastError());
-        const int hgrid = (int)std::min<int64_t>((psize + kBlock - 1) / kBlock, 1024);
-        colmask_hist_kernel<<<dim3(hgrid, num_parts), kBlock, 0, s>>>(colmask, num_cols, psize, hist);
-        LF_HIP(hipGetLastError());
+        if (h_colhist) {
+            const int hgrid = (int)std::min<int64_t>((psize + kBlock - 1) / kBlock, 1024);
+            colmask_hist_kernel<<<dim3(hgrid, num_parts), kBlock, 0, s>>>(colmask, num_cols, psize, hist);
+            LF_HIP(hipGetLastError());
+        }
     }
     LF_HIP(hipMemcpyAsync(h_stats, stats, stats_bytes, hipMemcpyDeviceToHost, s));
-    LF_HIP(hipMemcpyAsync(h_colhist, hist, hist_bytes, hipMemcpyDeviceToHost, s));
+    if (h_colhist) LF_HIP(hipMemcpyAsync(h_colhist, hist, hist_bytes, hipMemcpyDeviceToHost, s));
     LF_HIP(hipStreamSynchronize(s));
     return LF_OK;
 }

@@ -140,7 +140,9 @@ extern "C" int lf_search_bucket_config(const int64_t* h_stats, const int64_t* h_
                                        int32_t num_parts, int32_t width_limit, int32_t cfg_feat_size,
                                        int32_t cfg_num_parts, int32_t cost_model, int32_t* h_widths,
                                        int32_t* h_nwidths, double* h_trace_cost, int32_t* h_trace_len) {
-    LF_REQUIRE(h_stats && h_colhist && h_widths && h_nwidths, LF_ERR_INVALID, "null argument");
+    LF_REQUIRE(h_stats && h_widths && h_nwidths, LF_ERR_INVALID, "null argument");
+    LF_REQUIRE(h_colhist || cost_model == LF_COST_GFX950, LF_ERR_INVALID,
+               "the reference cost model needs the column histogram (null argument)");
     LF_REQUIRE(num_parts >= 1, LF_ERR_INVALID, "num_parts must be >= 1 (got %d)", num_parts);
     LF_REQUIRE(lf::is_pow2(width_limit) && width_limit <= (1 << (LF_MAX_CLASSES - 1)), LF_ERR_INVALID,
                "width_limit must be a power of two <= %d (got %d)", 1 << (LF_MAX_CLASSES - 1), width_limit);
@@ -151,7 +153,7 @@ extern "C" int lf_search_bucket_config(const int64_t* h_stats, const int64_t* h_
 
     for (int p = 0; p < num_parts; ++p) {
         const int64_t* st = h_stats + (size_t)p * LF_MAX_CLASSES * LF_STATS_FIELDS;
-        const int64_t* hist = h_colhist + (size_t)p * nmask;
+        const int64_t* hist = h_colhist ? h_colhist + (size_t)p * nmask : nullptr;
         int32_t* out_w = h_widths + (size_t)p * LF_MAX_CLASSES;
         double* trace = h_trace_cost ? h_trace_cost + (size_t)p * (LF_MAX_CLASSES + 1) : nullptr;
         int ntrace = 0;

@@ -126,23 +126,24 @@ def _cost_model_id(cfg) -> int:
 
 
 # --------------------------------------------------------------------------- search
-def bucket_statistics(g, num_parts: int, width_limit: int = WIDTH_LIMIT):
+def bucket_statistics(g, num_parts: int, width_limit: int = WIDTH_LIMIT, with_columns: bool = True):
     """Per-partition, per-width-class statistics of the initial bucketing
     (what get_init_buckets, format_algos.py:819-900, collects), computed on the GPU.
 
     Returns (stats, colhist): stats[p][k] = (cost-model rows, nnz, distinct rows, 0) for
-    width 2**k; colhist[p][m] = number of columns whose set of touching classes is mask m."""
+    width 2**k; colhist[p][m] = number of columns whose set of touching classes is mask m
+    (None with ``with_columns=False``: the gfx950 cost model does not use column sets)."""
     torch = _torch()
     lib = _lib.load()
     dev = _device_csr(g)
     stats = np.zeros((num_parts, _lib.LF_MAX_CLASSES, _lib.LF_STATS_FIELDS), dtype=np.int64)
-    hist = np.zeros((num_parts, 1 << _lib.LF_MAX_CLASSES), dtype=np.int64)
+    hist = np.zeros((num_parts, 1 << _lib.LF_MAX_CLASSES), dtype=np.int64) if with_columns else None
     nbytes = lib.lf_stats_workspace_bytes(dev.num_rows, dev.num_cols, num_parts)
     ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device="cuda")
     _lib.check(lib.lf_bucket_stats(_lib.ptr(dev.indptr), _lib.ptr(dev.indices), _lib.ptr(dev.seg_deg(num_parts)),
                                    dev.num_rows, dev.num_cols, num_parts, width_limit,
                                    _lib.ptr(ws), nbytes, _lib.np_ptr(stats, C.c_int64),
-                                   _lib.np_ptr(hist, C.c_int64), _stream()))
+                                   _lib.np_ptr(hist, C.c_int64) if with_columns else None, _stream()))
     return stats, hist
 
 
@@ -152,14 +153,14 @@ def search_from_statistics(stats, hist, cost_model_config, width_limit: int = WI
     lib = _lib.load()
     num_parts = stats.shape[0]
     stats = np.ascontiguousarray(stats, dtype=np.int64)
-    hist = np.ascontiguousarray(hist, dtype=np.int64)
+    hist = np.ascontiguousarray(hist, dtype=np.int64) if hist is not None else None
     widths = np.zeros((num_parts, _lib.LF_MAX_CLASSES), dtype=np.int32)
     nwidths = np.zeros(num_parts, dtype=np.int32)
     trace = np.zeros((num_parts, _lib.LF_MAX_CLASSES + 1), dtype=np.float64)
     trace_len = np.zeros(num_parts, dtype=np.int32)
     _lib.check(lib.lf_search_bucket_config(
-        _lib.np_ptr(stats, C.c_int64), _lib.np_ptr(hist, C.c_int64), num_parts, width_limit,
-        int(cost_model_config.feat_size), int(cost_model_config.num_parts), _cost_model_id(cost_model_config),
+        _lib.np_ptr(stats, C.c_int64), _lib.np_ptr(hist, C.c_int64) if hist is not None else None,
+        num_parts, width_limit, int(cost_model_config.feat_size), int(cost_model_config.num_parts), _cost_model_id(cost_model_config),
         _lib.np_ptr(widths, C.c_int32), _lib.np_ptr(nwidths, C.c_int32),
         _lib.np_ptr(trace, C.c_double), _lib.np_ptr(trace_len, C.c_int32)))
     config = [[int(w) for w in widths[p, :nwidths[p]]] for p in range(num_parts)]
@@ -171,7 +172,8 @@ def search_from_statistics(stats, hist, cost_model_config, width_limit: int = WI
 def search_bucket_config(g, num_parts: int, cost_model_config) -> List[List[int]]:
     """Bucket widths per column partition (format_algos.py:988-1032)."""
     num_parts = int(num_parts)
-    stats, hist = bucket_statistics(g, num_parts)
+    needs_columns = _cost_model_id(cost_model_config) == _lib.LF_COST_REFERENCE
+    stats, hist = bucket_statistics(g, num_parts, with_columns=needs_columns)
     return search_from_statistics(stats, hist, cost_model_config)
 
 
