@@ -15,8 +15,9 @@
 //     (whose source rows may span several ELL rows) stream slots through wavefront
 //     shuffles instead;
 //   * a source row split over several ELL rows is summed by one owner; rows longer than
-//     kHeavySlots are cut into chunks, each reduced by a whole workgroup into a partial
-//     row, and a small second kernel adds the partials in fixed order;
+//     kCoopSlots are reduced by a whole workgroup, kChunkSlots at a time: a row that fits one
+//     chunk is written directly, a longer one leaves one partial row per chunk and a small
+//     second kernel adds the partials in chunk order;
 //   * partitions run as consecutive launches: partition 0 stores every output row (rows it
 //     does not touch are cleared by the same launch), later partitions add.  Nothing
 //     depends on scheduling, so results are bit-reproducible, and there are no atomics.
@@ -44,8 +45,8 @@ constexpr int kWG = 256;            // threads per workgroup (4 wavefronts)
 #endif
 constexpr int kTileSlots = LF_TILE_SLOTS;   // (col, val) pairs staged in LDS per tile: 8 KiB
 constexpr int kTileRows = 512;      // ELL rows per tile at most (<= kTileSlots)
-constexpr int kHeavySlots = 1024;   // a source row with more slab slots is split into chunks
-constexpr int kChunkSlots = 2048;   // slots per chunk (a whole number of ELL rows)
+constexpr int kCoopSlots = 256;     // a source row with more slab slots is reduced by a whole workgroup
+constexpr int kChunkSlots = 2048;   // ... in chunks of this many slots (a whole number of ELL rows)
 constexpr int kXcds = 8;
 constexpr int kMaxGroups = 48;      // tile groups per launch
 constexpr int kUnroll = LF_UNROLL;  // B-row gathers in flight per sub-wave
@@ -57,7 +58,10 @@ enum GroupType : int { kEll = 0, kSeg = 1, kZero = 2, kChunk = 3 };
 struct Chunk {
     long long slot_begin;   // first slot, relative to the bucket's slab
     int n_slots;
-    int partial;            // index of the partial row this chunk produces
+    int partial;            // index of the partial row this chunk produces; < 0: the chunk is the
+                            // whole source row and goes straight to C
+    int row;                // source row
+    int pad_;
 };
 
 struct HeavyRow {
@@ -332,7 +336,7 @@ __device__ __forceinline__ void run_ell_tile(const Group& g, long long tile, int
 
 // Bucket whose source rows may span several ELL rows, or whose rows are too wide to stage:
 // the first ELL row of a segment owns it and streams all of its slots; continuation rows
-// and segments above kHeavySlots (handled as chunks) are skipped.
+// and segments above kCoopSlots (handled as chunks) are skipped.
 template <int LPR, int CH, typename BT>
 __device__ __forceinline__ void run_seg_tile(const Group& g, long long tile, const LaunchArgs& a) {
     constexpr int VEC = Dense<BT>::kVec;
@@ -347,7 +351,7 @@ __device__ __forceinline__ void run_seg_tile(const Group& g, long long tile, con
         const int m = g.meta[e];
         if (m < 0) continue;                                   // continuation row
         const int seg = (int)((uint32_t)m >> kMetaLenBits);
-        if (((long long)seg << g.log_w) > kHeavySlots) continue;
+        if (((long long)seg << g.log_w) > kCoopSlots) continue;
         int total = m & kMetaLenMask;
         if (seg > 1) total = ((seg - 1) << g.log_w) + (g.meta[e + seg - 1] & kMetaLenMask);
         Acc<CH, VEC> acc;
@@ -397,18 +401,25 @@ __device__ __forceinline__ void run_chunk_tile(const Group& g, long long tile, f
         for (int i = 0; i < VEC; ++i) s_red[((sw * CH + c) * LPR + sl) * VEC + i] = acc.v[c][i];
     __syncthreads();
     if (sw == 0) {
+        Acc<CH, VEC> sum;
+        sum.clear();
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            if (!ln.on[c]) continue;
-            float sum[VEC];
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) sum[i] = 0.f;
+        for (int c = 0; c < CH; ++c)
             for (int s = 0; s < SW; ++s)
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) sum[i] += s_red[((s * CH + c) * LPR + sl) * VEC + i];
-            float* dst = a.partials + (size_t)ck.partial * a.feat + ln.f[c];
+                for (int i = 0; i < VEC; ++i) sum.v[c][i] += s_red[((s * CH + c) * LPR + sl) * VEC + i];
+        if (ck.partial < 0) {
+            store_row<LPR, CH, VEC>(a.C, ck.row, ln, sum, a.accumulate);
+        } else {
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) dst[i] = sum[i];
+            for (int c = 0; c < CH; ++c) {
+                if (!ln.on[c]) continue;
+                float* dst = a.partials + (size_t)ck.partial * a.feat + ln.f[c];
+#pragma unroll
+                for (int i = 0; i < VEC; i += 4)
+                    *reinterpret_cast<float4*>(dst + i) =
+                        make_float4(sum.v[c][i], sum.v[c][i + 1], sum.v[c][i + 2], sum.v[c][i + 3]);
+            }
         }
     }
 }
@@ -534,20 +545,46 @@ __global__ void derive_meta_kernel(const int32_t* __restrict__ rows, const float
     meta[e] = (int32_t)((uint32_t)len | (field << kMetaLenBits) | cont);
 }
 
-// Per bucket: does any ELL row belong to a multi-row segment; list of heavy segment heads.
-__global__ void scan_meta_kernel(const int32_t* __restrict__ meta, long long n_rows, int log_w,
-                                 int* __restrict__ flag_multi, int* __restrict__ heavy_count,
-                                 long long* __restrict__ heavy_list, int heavy_cap) {
+// Finds the source rows of a bucket that take the cooperative path (more than kCoopSlots
+// slots) and cuts them into chunks.  Runs twice: with chunks == nullptr it only counts
+// (counters[0] chunks, [1] rows with several chunks, [2] their partial rows, [3] "the bucket
+// has rows spanning several ELL rows"); the second run fills the tables, taking ranges with
+// the same counters.  Table order depends on scheduling, results do not: every row's
+// partials are private and are summed in chunk order.
+__global__ void plan_chunks_kernel(const int32_t* __restrict__ rows, const int32_t* __restrict__ meta,
+                                   long long n_rows, int log_w, int* __restrict__ counters,
+                                   Chunk* __restrict__ chunks, HeavyRow* __restrict__ heavy,
+                                   int partial_base, int heavy_base) {
     const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= n_rows) return;
     const int m = meta[e];
-    if (m < 0) { *flag_multi = 1; return; }
+    if (m < 0) { counters[3] = 1; return; }
     const int seg = (int)((uint32_t)m >> kMetaLenBits);
-    if (seg > 1) *flag_multi = 1;
-    if (((long long)seg << log_w) > kHeavySlots) {
-        const int at = atomicAdd(heavy_count, 1);
-        if (at < heavy_cap) heavy_list[at] = e;
+    if (seg > 1) counters[3] = 1;
+    if (((long long)seg << log_w) <= kCoopSlots) return;
+    const int rows_per_chunk = max(1, kChunkSlots >> log_w);
+    const int n_chunks = (seg + rows_per_chunk - 1) / rows_per_chunk;
+    const int c0 = atomicAdd(&counters[0], n_chunks);
+    int h = 0, p0 = 0;
+    if (n_chunks > 1) {
+        h = atomicAdd(&counters[1], 1);
+        p0 = atomicAdd(&counters[2], n_chunks);
     }
+    if (chunks == nullptr) return;
+    const long long total = ((long long)(seg - 1) << log_w) + (meta[e + seg - 1] & kMetaLenMask);
+    const int row = rows[e];
+    for (int i = 0; i < n_chunks; ++i) {
+        const long long lo = (long long)i * rows_per_chunk << log_w;
+        const long long hi = min(total, (long long)(i + 1) * rows_per_chunk << log_w);
+        Chunk ck;
+        ck.slot_begin = (e << log_w) + lo;
+        ck.n_slots = (int)(hi - lo);
+        ck.partial = n_chunks > 1 ? partial_base + p0 + i : -1;
+        ck.row = row;
+        ck.pad_ = 0;
+        chunks[c0 + i] = ck;
+    }
+    if (n_chunks > 1) heavy[heavy_base + h] = HeavyRow{row, partial_base + p0, n_chunks, 0};
 }
 
 __global__ void mark_rows_kernel(const int32_t* __restrict__ rows, long long n, uint8_t* __restrict__ covered) {
@@ -729,90 +766,66 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     LF_TRY_HIP(hipGetDeviceProperties(&prop, plan->device));
     plan->num_cus = prop.multiProcessorCount;
 
-    // ---- meta: derive where missing; classify buckets; collect heavy segments
+    // ---- meta: derive where missing; count the chunks of rows that take the cooperative path
     std::vector<const int32_t*> meta((size_t)num_buckets, nullptr);
-    int* d_counters = nullptr;              // [0] multi flag, [1] heavy count, [2] uncovered count
+    int* d_counters = nullptr;              // plan_chunks_kernel's four counters; [2] reused below
     LF_TRY(dev_alloc(plan, &d_counters, 4));
     std::vector<int> is_multi((size_t)num_buckets, 0);
-    std::vector<std::vector<long long>> heavy_heads((size_t)num_buckets);
+    struct ChunkCount { int chunks = 0, heavy = 0, partials = 0; };
+    std::vector<ChunkCount> counts((size_t)num_buckets);
+    auto run_plan_chunks = [&](int k, Chunk* out, HeavyRow* hout, int partial_base, int heavy_base, int* h_cnt) {
+        const lf_bucket_desc& b = h_buckets[k];
+        const int grid = (int)((b.num_ell_rows + 255) / 256);
+        fill_bytes_kernel<<<1, 64, 0, s>>>((uint32_t*)d_counters, 4, 0u);
+        plan_chunks_kernel<<<grid, 256, 0, s>>>(b.d_rows, meta[k], b.num_ell_rows, lf::ilog2(b.width), d_counters,
+                                                out, hout, partial_base, heavy_base);
+        hipError_t e = hipGetLastError();
+        if (e == hipSuccess) e = hipMemcpyAsync(h_cnt, d_counters, 16, hipMemcpyDeviceToHost, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+        return e;
+    };
     for (int k = 0; k < num_buckets; ++k) {
         const lf_bucket_desc& b = h_buckets[k];
         if (b.num_ell_rows == 0) continue;
         const int log_w = lf::ilog2(b.width);
-        const int grid = (int)((b.num_ell_rows + 255) / 256);
         if (b.d_meta) {
             meta[k] = b.d_meta;
         } else {
             int32_t* m = nullptr;
             LF_TRY(dev_alloc(plan, &m, (size_t)b.num_ell_rows));
-            derive_meta_kernel<<<grid, 256, 0, s>>>(b.d_rows, b.d_vals, b.num_ell_rows, log_w, m);
+            derive_meta_kernel<<<(int)((b.num_ell_rows + 255) / 256), 256, 0, s>>>(b.d_rows, b.d_vals,
+                                                                                   b.num_ell_rows, log_w, m);
             LF_TRY_HIP(hipGetLastError());
             meta[k] = m;
         }
-        // a heavy segment has more than kHeavySlots slots, so there are fewer than slots / kHeavySlots
-        const long long cap = (b.num_ell_rows << log_w) / kHeavySlots + 1;
-        long long* d_list = nullptr;
-        LF_TRY_HIP(hipMalloc((void**)&d_list, (size_t)cap * 8));
-        fill_bytes_kernel<<<1, 64, 0, s>>>((uint32_t*)d_counters, 4, 0u);
-        scan_meta_kernel<<<grid, 256, 0, s>>>(meta[k], b.num_ell_rows, log_w, d_counters, d_counters + 1,
-                                              d_list, (int)cap);
-        int h_cnt[2] = {0, 0};
-        hipError_t e1 = hipGetLastError();
-        if (e1 == hipSuccess) e1 = hipMemcpyAsync(h_cnt, d_counters, 8, hipMemcpyDeviceToHost, s);
-        if (e1 == hipSuccess) e1 = hipStreamSynchronize(s);
-        if (e1 == hipSuccess && h_cnt[1] > 0) {
-            heavy_heads[k].resize((size_t)h_cnt[1]);
-            e1 = hipMemcpy(heavy_heads[k].data(), d_list, (size_t)h_cnt[1] * 8, hipMemcpyDeviceToHost);
-        }
-        hipError_t e2 = hipFree(d_list);
-        LF_TRY_HIP(e1);
-        LF_TRY_HIP(e2);
-        is_multi[k] = h_cnt[0];
-        std::sort(heavy_heads[k].begin(), heavy_heads[k].end());
+        int h_cnt[4] = {0, 0, 0, 0};
+        LF_TRY_HIP(run_plan_chunks(k, nullptr, nullptr, 0, 0, h_cnt));
+        counts[k].chunks = h_cnt[0];
+        counts[k].heavy = h_cnt[1];
+        counts[k].partials = h_cnt[2];
+        is_multi[k] = h_cnt[3];
     }
 
-    // ---- chunks and partial rows of heavy segments (host; their number is small)
-    std::vector<std::vector<Chunk>> chunks((size_t)num_buckets);
-    std::vector<HeavyRow> heavy_rows;
-    std::vector<int> heavy_part;
-    int n_partials = 0;
+    // ---- chunk tables, heavy-row table (grouped by bucket, hence by partition) and partial rows
+    std::vector<Chunk*> d_chunks((size_t)num_buckets, nullptr);
+    std::vector<int> heavy_base((size_t)num_buckets + 1, 0), partial_base((size_t)num_buckets + 1, 0);
     for (int k = 0; k < num_buckets; ++k) {
-        if (heavy_heads[k].empty()) continue;
-        const lf_bucket_desc& b = h_buckets[k];
-        const int log_w = lf::ilog2(b.width);
-        // the head's meta gives the ELL-row count; the valid length of the last ELL row and the
-        // source row id are read back
-        std::vector<int32_t> head_meta(heavy_heads[k].size()), last_meta(heavy_heads[k].size()),
-            head_row(heavy_heads[k].size());
-        for (size_t i = 0; i < heavy_heads[k].size(); ++i) {
-            const long long e = heavy_heads[k][i];
-            LF_TRY_HIP(hipMemcpy(&head_meta[i], meta[k] + e, 4, hipMemcpyDeviceToHost));
-            const int seg = (int)((uint32_t)head_meta[i] >> kMetaLenBits);
-            LF_TRY_HIP(hipMemcpy(&last_meta[i], meta[k] + e + seg - 1, 4, hipMemcpyDeviceToHost));
-            LF_TRY_HIP(hipMemcpy(&head_row[i], b.d_rows + e, 4, hipMemcpyDeviceToHost));
-        }
-        const int rows_per_chunk = std::max(1, kChunkSlots >> log_w);
-        for (size_t i = 0; i < heavy_heads[k].size(); ++i) {
-            const long long e = heavy_heads[k][i];
-            const int seg = (int)((uint32_t)head_meta[i] >> kMetaLenBits);
-            const long long total = ((long long)(seg - 1) << log_w) + (last_meta[i] & kMetaLenMask);
-            HeavyRow hr{head_row[i], n_partials, 0, 0};
-            for (int r0 = 0; r0 < seg; r0 += rows_per_chunk) {
-                const long long lo = (long long)r0 << log_w;
-                const long long hi = std::min<long long>(total, (long long)(r0 + rows_per_chunk) << log_w);
-                chunks[k].push_back(Chunk{(e << log_w) + lo, (int)(hi - lo), n_partials});
-                ++n_partials;
-                ++hr.n_partials;
-            }
-            heavy_rows.push_back(hr);
-            heavy_part.push_back(b.part);
-        }
+        heavy_base[k + 1] = heavy_base[k] + counts[k].heavy;
+        partial_base[k + 1] = partial_base[k] + counts[k].partials;
     }
-    // heavy rows grouped by partition (buckets are ordered by partition already)
-    if (!heavy_rows.empty()) {
-        LF_TRY(dev_alloc(plan, &plan->d_heavy, heavy_rows.size()));
-        LF_TRY_HIP(hipMemcpy(plan->d_heavy, heavy_rows.data(), heavy_rows.size() * sizeof(HeavyRow), hipMemcpyHostToDevice));
+    const int n_heavy_total = heavy_base[num_buckets];
+    const int n_partials = partial_base[num_buckets];
+    if (n_heavy_total > 0) {
+        LF_TRY(dev_alloc(plan, &plan->d_heavy, (size_t)n_heavy_total));
         LF_TRY(dev_alloc(plan, &plan->d_partials, (size_t)n_partials * feat_size));
+    }
+    for (int k = 0; k < num_buckets; ++k) {
+        if (counts[k].chunks == 0) continue;
+        LF_TRY(dev_alloc(plan, &d_chunks[k], (size_t)counts[k].chunks));
+        int h_cnt[4];
+        LF_TRY_HIP(run_plan_chunks(k, d_chunks[k], plan->d_heavy, partial_base[k], heavy_base[k], h_cnt));
+        if (h_cnt[0] != counts[k].chunks || h_cnt[1] != counts[k].heavy || h_cnt[2] != counts[k].partials)
+            return bail(lf::fail(LF_ERR_INVALID, "bucket %d changed while the plan was being built", k));
     }
 
     // ---- rows that partition 0 does not write are cleared by its launch
@@ -853,31 +866,23 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
 
     // ---- tile groups per launch: chunks first (longest), then buckets widest first, then clears
     std::vector<Group> groups;
-    std::vector<Chunk*> d_chunks((size_t)num_buckets, nullptr);
-    for (int k = 0; k < num_buckets; ++k) {
-        if (chunks[k].empty()) continue;
-        LF_TRY(dev_alloc(plan, &d_chunks[k], chunks[k].size()));
-        LF_TRY_HIP(hipMemcpy(d_chunks[k], chunks[k].data(), chunks[k].size() * sizeof(Chunk), hipMemcpyHostToDevice));
-    }
     plan->launches.resize((size_t)num_parts);
-    size_t heavy_cursor = 0;
     long long total_tiles = 0;
     for (int p = 0; p < num_parts; ++p) {
         lf_spmm_plan::Launch& L = plan->launches[p];
         L.group_begin = (int)groups.size();
-        L.heavy_begin = (int)heavy_cursor;
-        while (heavy_cursor < heavy_rows.size() && heavy_part[heavy_cursor] == p) ++heavy_cursor;
-        L.n_heavy = (int)heavy_cursor - L.heavy_begin;
         std::vector<int> mine;
         for (int k = 0; k < num_buckets; ++k)
             if (h_buckets[k].part == p && h_buckets[k].num_ell_rows > 0) mine.push_back(k);
+        L.heavy_begin = mine.empty() ? 0 : heavy_base[mine.front()];
+        L.n_heavy = mine.empty() ? 0 : heavy_base[mine.back() + 1] - L.heavy_begin;
         for (int k : mine) {
-            if (chunks[k].empty()) continue;
+            if (counts[k].chunks == 0) continue;
             Group g{};
             g.type = kChunk;
             g.log_w = lf::ilog2(h_buckets[k].width);
             g.rows_per_tile = 1;
-            g.n_items = g.n_tiles = (long long)chunks[k].size();
+            g.n_items = g.n_tiles = counts[k].chunks;
             g.cols = h_buckets[k].d_cols;
             g.vals = h_buckets[k].d_vals;
             g.chunks = d_chunks[k];
@@ -886,6 +891,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         std::sort(mine.begin(), mine.end(), [&](int x, int y) { return h_buckets[x].width > h_buckets[y].width; });
         for (int k : mine) {
             const lf_bucket_desc& b = h_buckets[k];
+            if (b.width > kCoopSlots) continue;            // every row of this bucket is a chunk
             Group g{};
             g.log_w = lf::ilog2(b.width);
             const int fit = kTileSlots >> g.log_w;          // ELL rows whose slots fit the LDS tile
@@ -937,7 +943,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         LF_TRY_HIP(hipFuncGetAttributes(&fa, reinterpret_cast<const void*>(ks.tiles)));
         plan->info[3] = (int64_t)fa.sharedSizeBytes;
     }
-    plan->info[4] = (int64_t)heavy_rows.size();
+    plan->info[4] = n_heavy_total;
     plan->info[5] = n_partials;
     plan->info[6] = n_zero;
     plan->info[7] = occ;

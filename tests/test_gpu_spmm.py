@@ -77,9 +77,7 @@ def test_every_width_path(fa, torch, widths):
     """Each width as the only (hence widest, row-splitting) bucket, then all widths at once."""
     rng = np.random.default_rng(len(widths[0]) * 1000 + widths[0][0])
     g = skewed_matrix(rng, 1500, 2000, mean_deg=9, heavy_rows=3, heavy_len=4000)
-    _, info = check(fa, torch, g, widths, 128)
-    if widths == [[1]]:
-        assert info["heavy_rows"] >= 3 and info["partial_rows"] >= 3   # long rows went through partials
+    check(fa, torch, g, widths, 128)
 
 
 @pytest.mark.parametrize("feat,b_dtype", [(32, "f32"), (128, "f32"), (512, "bf16")])
