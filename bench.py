@@ -86,6 +86,64 @@ def cpu_baseline(wl, B_host, feat, budget_s=20.0):
     }, out, take
 
 
+def bench_bsr(args):
+    """Block-sparse fp16 side path (bench_bsrmm's kernel): random 32 x 32 block structure."""
+    import scipy.sparse as sp
+    import torch
+    from liteform_ae_amd import format_algos as fa
+
+    feat = args.feat or 128
+    mb = nb = max(8, int(round(32768 * args.scale)))
+    per_row = 8
+    rng = np.random.default_rng(1006)
+    cols = np.sort(rng.integers(0, nb, size=(mb, per_row)), axis=1)
+    keep = np.ones_like(cols, dtype=bool)
+    keep[:, 1:] = cols[:, 1:] != cols[:, :-1]
+    indptr = np.zeros(mb + 1, dtype=np.int32)
+    indptr[1:] = np.cumsum(keep.sum(1))
+    indices = cols[keep].astype(np.int32)
+    nnzb = len(indices)
+    dev = fa._DeviceBSR.__new__(fa._DeviceBSR)
+    dev.block_size, dev.mb, dev.nb, dev.nnzb = 32, mb, nb, nnzb
+    dev.indptr = torch.from_numpy(indptr).cuda()
+    dev.indices = torch.from_numpy(indices).cuda()
+    dev.data = (torch.rand(nnzb * 1024, device="cuda") - 0.5).to(torch.float16)
+    x = (torch.rand((nb * 32, feat), device="cuda") - 0.5).to(torch.float16)
+    for _ in range(args.warmup):
+        fa.spmm_bsr(dev, x)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        y = fa.spmm_bsr(dev, x)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    ev = []
+    for _ in range(args.steps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fa.spmm_bsr(dev, x)
+        b.record()
+        b.synchronize()
+        ev.append(a.elapsed_time(b))
+    kernel_ms = float(np.mean(ev))
+    flops = 2.0 * nnzb * 1024 * feat
+    algo = nnzb * 2048 + nnzb * 4 + (mb + 1) * 4 + nb * 32 * feat * 2 + mb * 32 * feat * 2
+    gath = nnzb * 2048 + nnzb * 4 + (mb + 1) * 4 + nnzb * 32 * feat * 2 + mb * 32 * feat * 2
+    print(json.dumps({
+        "metric": "BSR (32x32, fp16) SpMM GFLOP/s", "value": round(flops / (ms * 1e-3) / 1e9, 1), "unit": "GFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 in, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": f"bsr: {mb * 32} x {nb * 32}, {nnzb} dense 32x32 blocks (~{per_row} per block row)",
+                   "feat_size": feat},
+        "roofline": {"bound": "hbm", "achieved": round(algo / (kernel_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(algo / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes": algo,
+                     "gather_bytes": gath, "gather_GBps": round(gath / (kernel_ms * 1e-3) / 1e9, 1),
+                     "mfma_TFLOPs": round(flops / (kernel_ms * 1e-3) / 1e12, 1)},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -119,6 +177,8 @@ def main():
         sys.exit(2)
     _lib.load()
     torch.cuda.set_device(0)
+    if args.workload == "bsr":
+        return bench_bsr(args)
 
     t0 = time.perf_counter()
     wl = make_workload(args.workload, args.scale)

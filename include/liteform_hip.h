@@ -199,6 +199,15 @@ int lf_csr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const float* 
                 int64_t num_rows, int64_t num_cols, int32_t feat_size, int32_t b_dtype,
                 const void* d_B, float* d_C, lf_stream_t stream);
 
+/* Block-sparse SpMM on the matrix cores, the counterpart of bench_bsrmm's kernel
+ * (format_algos.py:1182-1643): Y = A_bsr . X with 32 x 32 fp16 blocks (scipy BSR layout:
+ * indptr [num_block_rows + 1], indices [nnz blocks], data [nnz blocks][32][32] row-major),
+ * X [num_block_cols * 32][feat] fp16, Y [num_block_rows * 32][feat] fp16, fp32 accumulation
+ * (the reference accumulates in fp16).  feat_size must be a multiple of 8. */
+int lf_bsr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const void* d_data,
+                int64_t num_block_rows, int64_t num_block_cols, int32_t block_size,
+                int32_t feat_size, const void* d_X, void* d_Y, lf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -15,7 +15,7 @@ def __getattr__(name):
     # format_algos needs torch and the HIP library; load it on first use so that
     # the container classes stay importable on their own.
     if name in ("CostModelSettings", "search_bucket_config", "build_hyb_format",
-                "bench_hyb_with_config", "bench_naive", "HybFormat", "build_hyb_format_device"):
+                "bench_hyb_with_config", "bench_naive", "bench_bsrmm", "HybFormat", "build_hyb_format_device"):
         from . import format_algos
         return getattr(format_algos, name)
     raise AttributeError(name)

@@ -33,7 +33,7 @@ from . import _lib
 from .format_matrix_market import MTX, Bucket  # noqa: F401  (re-exported like the reference)
 
 __all__ = ["build_hyb_format", "bench_hyb_with_config", "search_bucket_config",
-           "CostModelSettings", "bench_naive",
+           "CostModelSettings", "bench_bsrmm", "bench_naive", "spmm_bsr",
            "build_hyb_format_device", "HybFormat", "HybSpMM", "spmm_hyb", "spmm_csr",
            "guess_num_partitions", "choose_num_partitions"]
 
@@ -470,6 +470,66 @@ def bench_hyb_with_config(g, x, y_ndarray, feat_size=128, bucket_widths=[], buck
         plan.close()
     print("cell exe time: {:.6f} ms".format(dur))
     return dur
+
+
+class _DeviceBSR:
+    """scipy BSR arrays on the GPU: int32 index arrays, fp16 blocks."""
+
+    def __init__(self, bsr_mat, block_size: int):
+        torch = _torch()
+        if tuple(bsr_mat.blocksize) != (block_size, block_size):
+            raise ValueError(f"matrix has blocks {bsr_mat.blocksize}, expected {(block_size, block_size)}")
+        if not bsr_mat.has_sorted_indices:
+            bsr_mat = bsr_mat.copy()
+            bsr_mat.sort_indices()
+        self.block_size = block_size
+        self.mb = bsr_mat.shape[0] // block_size
+        self.nb = bsr_mat.shape[1] // block_size
+        self.nnzb = int(len(bsr_mat.indices))
+        self.indptr = torch.from_numpy(np.ascontiguousarray(bsr_mat.indptr, dtype=np.int32)).cuda()
+        self.indices = torch.from_numpy(np.ascontiguousarray(bsr_mat.indices, dtype=np.int32)).cuda()
+        self.data = torch.from_numpy(np.ascontiguousarray(bsr_mat.data, dtype=np.float16).reshape(-1)).cuda()
+
+
+def spmm_bsr(bsr, x, block_size: int = 32):
+    """Y = A_bsr . X on the matrix cores.  ``bsr`` is a scipy BSR matrix or a ``_DeviceBSR``;
+    ``x`` a CUDA fp16 tensor (cols, N).  Returns a CUDA fp16 tensor (rows, N)."""
+    torch = _torch()
+    lib = _lib.load()
+    dev = bsr if isinstance(bsr, _DeviceBSR) else _DeviceBSR(bsr, block_size)
+    feat = int(x.shape[1])
+    if x.dtype != torch.float16 or not x.is_cuda or not x.is_contiguous() or x.shape[0] != dev.nb * dev.block_size:
+        raise ValueError(f"x must be a contiguous CUDA fp16 tensor with {dev.nb * dev.block_size} rows")
+    y = torch.empty((dev.mb * dev.block_size, feat), dtype=torch.float16, device="cuda")
+    _lib.check(lib.lf_bsr_spmm(_lib.ptr(dev.indptr), _lib.ptr(dev.indices), _lib.ptr(dev.data), dev.mb, dev.nb,
+                               dev.block_size, feat, x.data_ptr(), y.data_ptr(), _stream()))
+    return y
+
+
+def bench_bsrmm(bsr_mat, x, block_size: int):
+    """Time the block-sparse fp16 kernel; returns the mean kernel time in ms
+    (format_algos.py:1562-1643).  ``x`` is a (cols, N) fp16 torch tensor on the host, as the
+    driver makes it (proc05.spmm.end-to-end.py:221)."""
+    torch = _torch()
+    dev = _DeviceBSR(bsr_mat, block_size)
+    xd = x.to(torch.float16).contiguous().cuda()
+    bench_bsrmm.last_output = spmm_bsr(dev, xd)
+    warmup, repeat = _timing_params()
+    flush = _flush_buffer()
+    for _ in range(warmup):
+        spmm_bsr(dev, xd)
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(repeat)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(repeat)]
+    for i in range(repeat):
+        if flush is not None:
+            flush.zero_()
+        starts[i].record()
+        spmm_bsr(dev, xd)
+        ends[i].record()
+    torch.cuda.synchronize()
+    avg_time = float(np.mean([s.elapsed_time(e) for s, e in zip(starts, ends)]))
+    print("bsrmm time: \t{:.5f}ms".format(avg_time))
+    return avg_time
 
 
 def bench_naive(g, x, y_ndarray, feat_size=128, coarsening_factor=2, check_correctness=False):

@@ -129,6 +129,19 @@ class MTX:
         """A @ B through scipy (format_matrix_market.py:89-99)."""
         return self.coo_mtx.tocsc().dot(B)
 
+    def tobsr(self, blocksize=None, copy=False):
+        """scipy BSR view (format_matrix_market.py:101-112)."""
+        return self.coo_mtx.tobsr(blocksize=blocksize, copy=copy)
+
+    def tobsr_with_padding(self, shape, blocksize=None):
+        """BSR matrix of the given (padded) shape with fp16-valued entries, shape % blocksize == 0
+        (format_matrix_market.py:115-136).  The reference stores the values as float16; scipy
+        1.15 no longer accepts that dtype in sparse containers, so the values are rounded to
+        fp16 and held as float32 (every value is exactly representable in fp16)."""
+        data = np.array(self.coo_mtx.data, dtype=np.float16).astype(np.float32)
+        ij = [self.coo_mtx.row, self.coo_mtx.col]
+        return sp.bsr_matrix((data, ij), blocksize=blocksize, shape=shape)
+
     def tocsr(self, copy=False):
         return self.coo_mtx.tocsr(copy=copy)
 

@@ -459,3 +459,15 @@ def spmm_from_hyb(rows_nd, cols_nd, vals_nd, num_rows: int, B: np.ndarray) -> np
             contrib = np.einsum("ew,ewn->en", np.asarray(vals, dtype=np.float64), B[cols])
             np.add.at(C, rows, contrib)
     return C
+
+
+def spmm_bsr_f64(bsr_mat, X: np.ndarray) -> np.ndarray:
+    """Block-sparse product in float64: what bench_bsrmm's kernel computes
+    (format_algos.py:1182-1216: C[i, bi, f] = sum_j sum_bj A[i, j, bi, bj] * B[j, bj, f]),
+    through scipy's BSR @ dense with both operands widened first."""
+    return bsr_mat.astype(np.float64) @ np.asarray(X, dtype=np.float64)
+
+
+def spmm_bsr_abs_bound(bsr_mat, X: np.ndarray) -> np.ndarray:
+    """sum |a| |x| per output element, the scale of the accumulation error."""
+    return abs(bsr_mat.astype(np.float64)) @ np.abs(np.asarray(X, dtype=np.float64))
