@@ -27,11 +27,38 @@ from .format_matrix_market import MTX
 FEAT_SIZES = (32, 64, 128, 256, 512)        # proc05.spmm.end-to-end.py:141
 
 
+def _run_block_or_csr(g, fa, feat, fmt_name):
+    """The reference's branch for matrices its selector sends away from CELL
+    (proc05.spmm.end-to-end.py:191-261): pad to a multiple of 32 and run the fp16 BSR kernel;
+    if that fails, or when CSR is asked for, run the row-parallel CSR kernel."""
+    import torch
+    bsize = 32                                                         # proc05:205
+    num_src, num_dst = g.num_src_nodes(), g.num_dst_nodes()
+    side = -(-max(num_src, num_dst) // bsize) * bsize                  # proc05:198-210
+    if fmt_name == "BSR":
+        try:
+            bsr_weight = g.tobsr_with_padding(shape=(side, side), blocksize=(bsize, bsize))
+            x = torch.rand(bsr_weight.shape[1], feat).half()           # proc05:221
+            return "BSR", fa.bench_bsrmm(bsr_weight, x, block_size=bsize)
+        except Exception as e:                                         # proc05:232-234
+            print(e, file=sys.stderr)
+            print(f"name {g.name} in BSR failed. Do CSR then.")
+    try:
+        x = torch.rand((num_dst, feat))                                # proc05:239
+        y_ndarray = g.dot(x.numpy())
+        return "CSR", fa.bench_naive(g, x, y_ndarray, feat_size=feat, coarsening_factor=2)
+    except Exception as e2:                                            # proc05:254-261
+        print(e2, file=sys.stderr)
+        return "CRASHED", 0
+
+
 def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="reference",
-                   check_correctness=False, out_csv=None, keep_values=False):
+                   check_correctness=False, out_csv=None, keep_values=False, select_format=None):
     """Runs the flow for an iterable of MTX objects and returns a pandas DataFrame with the
     reference's columns.  ``num_parts``: None = measure per (matrix, feature size); an int;
-    or a callable ``(g, feat_size) -> int``."""
+    or a callable ``(g, feat_size) -> int``.  ``select_format``: None = CELL for every
+    matrix; or a callable ``g -> "CELL" | "BSR" | "CSR"`` standing in for the reference's
+    format-selection model (proc05.spmm.end-to-end.py:133)."""
     import pandas as pd
     import torch
 
@@ -42,7 +69,20 @@ def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="
                              "time_compose(ms)", "GFLOP/s", "bucket_config")}
     for g in matrices:
         print(f"\nGo to name {g.name} ...")
-        fmt_name, time_select = "CELL", 0.0
+        t0 = time.perf_counter()
+        fmt_name = select_format(g) if select_format else "CELL"
+        time_select = time.perf_counter() - t0
+        if fmt_name != "CELL":
+            for feat in feat_sizes:
+                ran_as, exe_time = _run_block_or_csr(g, fa, feat, fmt_name)
+                row = {"name": g.name, "format": ran_as, "feat_size": feat, "num_parts": 0,
+                       "time_select(s)": time_select, "time_num_parts(s)": 0, "time_bucket(s)": 0,
+                       "time_exe_our(ms)": exe_time, "time_compose(ms)": float("nan"),
+                       "GFLOP/s": 2.0 * g.num_edges() * feat / (exe_time * 1e-3) / 1e9 if exe_time > 0 else 0.0,
+                       "bucket_config": ""}
+                for k, v in row.items():
+                    table[k].append(v)
+            continue
         for feat in feat_sizes:
             t0 = time.perf_counter()
             if num_parts is None:
@@ -104,6 +144,8 @@ def main(argv=None):
     ap.add_argument("--feat", type=int, nargs="*", default=list(FEAT_SIZES))
     ap.add_argument("--num-parts", type=int, default=0, help="0 = choose by measurement")
     ap.add_argument("--cost-model", default="reference", choices=["reference", "gfx950"])
+    ap.add_argument("--format", default="CELL", choices=["CELL", "BSR", "CSR"],
+                    help="format to run every matrix in (the reference chooses it with a model)")
     ap.add_argument("--check", action="store_true", help="compare with scipy (rtol 1e-4) as the reference can")
     ap.add_argument("--csv", default="", help="write the table to this file")
     args = ap.parse_args(argv)
@@ -118,7 +160,8 @@ def main(argv=None):
         ap.print_help(sys.stderr)
         return 2
     run_end_to_end(mats, feat_sizes=args.feat, num_parts=args.num_parts or None, cost_model=args.cost_model,
-                   check_correctness=args.check, out_csv=args.csv or None)
+                   check_correctness=args.check, out_csv=args.csv or None,
+                   select_format=(lambda g: args.format) if args.format != "CELL" else None)
     return 0
 
 

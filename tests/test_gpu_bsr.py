@@ -98,3 +98,20 @@ def test_reference_driver_branch(fa, torch):
     assert (np.abs(y - ref) <= 2.0 ** -10 * np.abs(ref) + 1e-5 * O.spmm_bsr_abs_bound(bsr_weight, x.numpy()) + 1e-7).all()
     with pytest.raises(NotImplementedError):
         fa.bench_bsrmm(g.tobsr_with_padding(shape=(1008, 1008), blocksize=(16, 16)), torch.rand(1008, 64).half(), 16)
+
+
+def test_driver_block_and_csr_branches(fa, torch):
+    """proc05.spmm.end-to-end.py:191-261 through the driver: BSR, CSR, and the table's columns."""
+    from liteform_ae_amd import driver
+    from liteform_ae_amd.format_matrix_market import MTX
+    rng = np.random.default_rng(6)
+    n = 700
+    key = np.unique(rng.integers(0, n, size=5000) * n + rng.integers(0, n, size=5000))
+    g = MTX.from_coo(key // n, key % n, (n, n), name="toy")
+    import os
+    os.environ["LF_REPEAT"] = "2"
+    os.environ["LF_WARMUP"] = "1"
+    df = driver.run_end_to_end([g], feat_sizes=(32, 64), select_format=lambda m: "BSR")
+    assert (df["format"] == "BSR").all() and (df["time_exe_our(ms)"] > 0).all() and (df["num_parts"] == 0).all()
+    df = driver.run_end_to_end([g], feat_sizes=(64,), select_format=lambda m: "CSR")
+    assert (df["format"] == "CSR").all() and (df["time_exe_our(ms)"] > 0).all()
