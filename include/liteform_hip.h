@@ -199,6 +199,18 @@ int lf_csr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const float* 
                 int64_t num_rows, int64_t num_cols, int32_t feat_size, int32_t b_dtype,
                 const void* d_B, float* d_C, lf_stream_t stream);
 
+/* COO -> canonical CSR on the GPU: entries sorted by (row, column), duplicates added up,
+ * row pointer built - what the reference's container does with scipy's coo.tocsr() on every
+ * CSR request (format_matrix_market.py:74-76).  d_coo_val NULL = all ones (the reference's
+ * matrices, format_matrix_market.py:54, 63-64).  Outputs: d_indptr [num_rows + 1], d_indices
+ * and d_values with room for nnz entries; *h_nnz_out = entries left after merging duplicates.
+ * Synchronises the stream. */
+size_t lf_coo_to_csr_workspace_bytes(int64_t nnz, int64_t num_rows, int64_t num_cols);
+int lf_coo_to_csr(const int32_t* d_coo_row, const int32_t* d_coo_col, const float* d_coo_val, int64_t nnz,
+                  int64_t num_rows, int64_t num_cols, void* d_workspace, size_t workspace_bytes,
+                  int32_t* d_indptr, int32_t* d_indices, float* d_values, int64_t* h_nnz_out,
+                  lf_stream_t stream);
+
 /* Block-sparse SpMM on the matrix cores, the counterpart of bench_bsrmm's kernel
  * (format_algos.py:1182-1643): Y = A_bsr . X with 32 x 32 fp16 blocks (scipy BSR layout:
  * indptr [num_block_rows + 1], indices [nnz blocks], data [nnz blocks][32][32] row-major),

@@ -67,6 +67,8 @@ SIGNATURES = {
     "lf_spmm_info": (C.c_int, [vp, i64p]),
     "lf_spmm_time_ms": (C.c_int, [vp, vp, vp, C.c_int32, C.c_int32, vp, C.c_size_t, f32p, vp]),
     "lf_csr_spmm": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int32, C.c_int32, vp, vp, vp]),
+    "lf_coo_to_csr_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int64]),
+    "lf_coo_to_csr": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int64, vp, C.c_size_t, vp, vp, vp, i64p, vp]),
     "lf_bsr_spmm": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int32, C.c_int32, vp, vp, vp]),
 }
 

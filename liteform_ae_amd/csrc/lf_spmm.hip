@@ -850,7 +850,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         if (e == hipSuccess) e = hipStreamSynchronize(s);
         if (e == hipSuccess && n_zero > 0) {
             int rc = dev_alloc(plan, &d_zero_rows, (size_t)n_zero);
-            if (rc != LF_OK) { hipFree(d_cov); return bail(rc); }
+            if (rc != LF_OK) { (void)hipFree(d_cov); return bail(rc); }
             fill_bytes_kernel<<<1, 64, 0, s>>>((uint32_t*)d_counters, 4, 0u);
             collect_uncovered_kernel<<<rgrid, 256, 0, s>>>(d_cov, num_rows, d_counters + 2, d_zero_rows);
             e = hipGetLastError();
@@ -1044,8 +1044,8 @@ int lf_spmm_time_ms(lf_spmm_plan* plan, const void* d_B, float* d_C, int32_t war
         if (e == hipSuccess) e = hipEventElapsedTime(&h_ms[i], t0, t1);
         if (e != hipSuccess) rc = lf::fail(LF_ERR_HIP, "timing failed: %s", hipGetErrorString(e));
     }
-    hipEventDestroy(t0);
-    hipEventDestroy(t1);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
     return rc;
 }
 

@@ -67,23 +67,42 @@ def _stream():
 
 
 class _DeviceCSR:
-    """CSR arrays of a matrix on the GPU (int32 indices, float32 values)."""
+    """CSR arrays of a matrix on the GPU (int32 indices, float32 values), made from the
+    container's COO triplets by lf_coo_to_csr: sorted columns, duplicates summed - the GPU
+    counterpart of the scipy conversion behind adj_tensors("csr")
+    (format_matrix_market.py:74-76)."""
 
     def __init__(self, g):
         torch = _torch()
-        indptr, indices, data = g.adj_tensors("csr")
+        lib = _lib.load()
+        coo = g.coo_mtx
         self.num_rows = int(g.num_src_nodes())
         self.num_cols = int(g.num_dst_nodes())
-        self.nnz = int(len(indices))
-        if self.nnz >= 2**31:
-            raise NotImplementedError("matrices with 2^31 or more stored entries are not supported")
-        self.indptr = torch.from_numpy(np.ascontiguousarray(indptr, dtype=np.int32)).cuda()
-        self.indices = torch.from_numpy(np.ascontiguousarray(indices, dtype=np.int32)).cuda()
-        self.values = torch.from_numpy(np.ascontiguousarray(data, dtype=np.float32)).cuda()
-        self.all_ones = bool(np.all(np.asarray(data) == 1))
         # The reference counts degrees from raw COO triplets (format_algos.py:250, 846); they
         # differ from the CSR row lengths only when the COO holds duplicates.
         self.coo_nnz = int(g.num_edges())
+        if self.coo_nnz >= 2**31:
+            raise NotImplementedError("matrices with 2^31 or more stored entries are not supported")
+        row = torch.from_numpy(np.ascontiguousarray(coo.row, dtype=np.int32)).cuda()
+        col = torch.from_numpy(np.ascontiguousarray(coo.col, dtype=np.int32)).cuda()
+        data = np.asarray(coo.data)
+        ones = bool(np.all(data == 1))
+        val = None if ones else torch.from_numpy(np.ascontiguousarray(data, dtype=np.float32)).cuda()
+        n = max(self.coo_nnz, 1)
+        self.indptr = torch.empty(self.num_rows + 1, dtype=torch.int32, device="cuda")
+        indices = torch.empty(n, dtype=torch.int32, device="cuda")
+        values = torch.empty(n, dtype=torch.float32, device="cuda")
+        nbytes = lib.lf_coo_to_csr_workspace_bytes(self.coo_nnz, self.num_rows, self.num_cols)
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device="cuda")
+        out = C.c_int64(0)
+        _lib.check(lib.lf_coo_to_csr(_lib.ptr(row), _lib.ptr(col), _lib.ptr(val), self.coo_nnz, self.num_rows,
+                                     self.num_cols, _lib.ptr(ws), nbytes, _lib.ptr(self.indptr),
+                                     _lib.ptr(indices), _lib.ptr(values), C.byref(out), _stream()))
+        self.nnz = int(out.value)
+        self.indices = indices[:self.nnz]
+        self.values = values[:self.nnz]
+        # duplicates of unit entries add up to 2, 3, ...: only a duplicate-free unit matrix is "all ones"
+        self.all_ones = ones and self.nnz == self.coo_nnz
         self._g = g
         self._seg_deg = {}
 

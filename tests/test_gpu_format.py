@@ -131,3 +131,28 @@ def test_workload_shapes_scaled(fa):
         cfg = fa.search_bucket_config(g, parts, fa.CostModelSettings(wl.feat_size, parts))
         assert cfg == O.search_bucket_config(g, parts, O.OracleCostModelSettings(wl.feat_size, parts)), name
         assert_hyb_equal(fa.build_hyb_format(g, cfg), O.build_hyb_format_closed_form(g, cfg))
+
+
+def test_device_ingest_matches_scipy_tocsr(fa):
+    """lf_coo_to_csr against coo.tocsr() (format_matrix_market.py:74-76): unsorted triplets,
+    duplicates, empty rows, rectangular shapes."""
+    import scipy.sparse as sp
+    from liteform_ae_amd.format_matrix_market import MTX
+    rng = np.random.default_rng(17)
+    for (nr, nc, n, weighted) in ((1, 1, 1, False), (300, 500, 4000, False), (2000, 70, 30000, True),
+                                  (5, 100000, 2000, True), (100000, 3, 50000, False)):
+        r = rng.integers(0, nr, size=n)
+        c = rng.integers(0, nc, size=n)
+        d = rng.uniform(-1, 1, size=n) if weighted else None
+        g = MTX.from_coo(r, c, (nr, nc), data=d)
+        dev = fa._DeviceCSR(g)
+        want = g.coo_mtx.tocsr()
+        want.sum_duplicates()
+        assert dev.nnz == want.nnz and dev.coo_nnz == n
+        np.testing.assert_array_equal(dev.indptr.cpu().numpy(), want.indptr)
+        np.testing.assert_array_equal(dev.indices.cpu().numpy(), want.indices)
+        np.testing.assert_allclose(dev.values.cpu().numpy(), want.data, rtol=1e-5, atol=1e-6)
+        assert dev.all_ones == (not weighted and want.nnz == n)
+    g = MTX.from_coo(np.zeros(0, np.int64), np.zeros(0, np.int64), (7, 9))
+    dev = fa._DeviceCSR(g)
+    assert dev.nnz == 0 and dev.indptr.cpu().numpy().tolist() == [0] * 8
