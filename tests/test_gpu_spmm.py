@@ -89,6 +89,15 @@ def test_very_long_rows_are_split_into_chunks(fa, torch, feat, b_dtype):
         assert info["heavy_rows"] >= 2 and info["partial_rows"] >= 2 * 8
 
 
+@pytest.mark.parametrize("feat,b_dtype", [(768, "f32"), (1024, "f32"), (1024, "bf16"), (32, "bf16"), (160, "f32")])
+def test_wide_and_odd_feature_sizes(fa, torch, feat, b_dtype):
+    """Several 16-byte chunks per lane (N > 256 fp32, N > 512 bf16) and lanes past the end."""
+    rng = np.random.default_rng(feat)
+    g = skewed_matrix(rng, 700, 900, mean_deg=6, heavy_rows=2, heavy_len=2500)
+    for widths in ([[1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024]], [[2, 16]]):
+        check(fa, torch, g, widths, feat, b_dtype, seed=feat)
+
+
 def test_bf16_dense_operand(fa, torch):
     rng = np.random.default_rng(5)
     g = skewed_matrix(rng, 2000, 3000, mean_deg=8, heavy_rows=3, heavy_len=2500)

@@ -333,3 +333,15 @@ def test_spmm_anchors():
     g = MTX(None)
     g.coo_mtx = a.tocoo()
     np.testing.assert_allclose(O.spmm_reference_f64(g, B), a.toarray() @ B, rtol=1e-12, atol=1e-12)
+
+
+def test_bsr_oracle_against_dense():
+    rng = np.random.default_rng(2)
+    blocks = rng.uniform(-1, 1, size=(5, 32, 32)).astype(np.float32)
+    a = sp.bsr_matrix((blocks, np.array([0, 2, 1, 0, 2]), np.array([0, 2, 3, 5])), shape=(96, 96))
+    x = rng.uniform(-1, 1, size=(96, 7))
+    np.testing.assert_allclose(O.spmm_bsr_f64(a, x), a.toarray().astype(np.float64) @ x, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(O.spmm_bsr_abs_bound(a, x), np.abs(a.toarray()).astype(np.float64) @ np.abs(x),
+                               rtol=1e-12, atol=1e-12)
+    eye = sp.identity(64, format="csr").tobsr(blocksize=(32, 32))
+    np.testing.assert_array_equal(O.spmm_bsr_f64(eye, x[:64]), x[:64])
