@@ -62,7 +62,7 @@ constexpr int kUnroll = LF_UNROLL;  // B-row gathers in flight per sub-wave
 constexpr uint32_t kMetaLenMask = 0x7FFu;
 constexpr int kMetaLenBits = 11;
 
-enum GroupType : int { kEll = 0, kSeg = 1, kZero = 2, kChunk = 3 };
+enum GroupType : int { kEll = 0, kSeg = 1, kZero = 2, kChunk = 3, kEllSeg = 4 };
 
 struct Chunk {
     long long slot_begin;   // first slot, relative to the bucket's slab
@@ -306,6 +306,51 @@ __device__ __forceinline__ void ell_tile_wide(const int2* s_pairs, const int2* s
     }
 }
 
+// Staged tile of a bucket whose source rows may span several consecutive ELL rows (the widest
+// bucket of a partition): the first ELL row of a segment owns it.  The part of the segment
+// inside the tile is read from LDS, a part that runs past the tile's end is streamed from
+// global memory.  Continuation rows and rows that take the cooperative path are skipped.
+template <int LPR, int CH, typename BT>
+__device__ __forceinline__ void ell_tile_segments(const Group& g, long long e0, const int2* s_pairs,
+                                                  const int2* s_rm, int n, const LaunchArgs& a, int sw, int sl) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int SW = kWG / LPR;
+    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const int log_w = g.log_w;
+    for (int r = sw; r < n; r += SW) {
+        const int2 rm = s_rm[r];
+        if (rm.y < 0) continue;                                  // continuation row
+        const int seg = (int)((uint32_t)rm.y >> kMetaLenBits);
+        if (((long long)seg << log_w) > kCoopSlots) continue;   // reduced by a whole workgroup
+        int total = rm.y & kMetaLenMask;
+        if (seg > 1) {
+            const int last = r + seg - 1;
+            const int last_meta = last < n ? s_rm[last].y : g.meta[e0 + last];
+            total = ((seg - 1) << log_w) + (last_meta & kMetaLenMask);
+        }
+        const int staged = min(total, (n - r) << log_w);
+        const int2* rp = s_pairs + (r << log_w);
+        const int c0 = rp[0].x;
+        Acc<CH, VEC> acc;
+        acc.clear();
+        for (int j = 0; j < staged; j += kUnroll) {
+            int c[kUnroll];
+            float v[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const bool in = j + u < staged;
+                const int2 cv = rp[in ? j + u : 0];
+                c[u] = in ? cv.x : c0;
+                v[u] = in ? __int_as_float(cv.y) : 0.f;
+            }
+            gather_fma<kUnroll, LPR, CH, BT>(a.B, ln, c, v, acc);
+        }
+        if (total > staged)
+            stream_slots<LPR, CH, BT>(g.cols, g.vals, ((e0 + r) << log_w) + staged, total - staged, a.B, ln, acc);
+        store_row<LPR, CH, VEC>(a.C, rm.x, ln, acc, a.accumulate);
+    }
+}
+
 template <int LPR, int CH, typename BT>
 __device__ __forceinline__ void run_ell_tile(const Group& g, long long tile, int2* s_pairs, int2* s_rm,
                                              const LaunchArgs& a) {
@@ -330,6 +375,10 @@ __device__ __forceinline__ void run_ell_tile(const Group& g, long long tile, int
     for (int i = tid; i < n; i += kWG) s_rm[i] = make_int2(g.rows[e0 + i], g.meta[e0 + i]);
     __syncthreads();
     const int sw = tid / LPR, sl = tid % LPR;
+    if (g.type == kEllSeg) {
+        ell_tile_segments<LPR, CH, BT>(g, e0, s_pairs, s_rm, n, a, sw, sl);
+        return;
+    }
     switch (g.log_w) {
         case 0: ell_tile_narrow<1, LPR, CH, BT>(s_pairs, s_rm, n, a, sw, sl); break;
         case 1: ell_tile_narrow<2, LPR, CH, BT>(s_pairs, s_rm, n, a, sw, sl); break;
@@ -459,7 +508,8 @@ spmm_partition_kernel(LaunchArgs a) {
         if (v < hi - lo) {
             const long long tile = lo + v;
             switch (g.type) {
-                case kEll: run_ell_tile<LPR, CH, BT>(g, tile, s_pairs, s_rm, a); break;
+                case kEll:
+                case kEllSeg: run_ell_tile<LPR, CH, BT>(g, tile, s_pairs, s_rm, a); break;
                 case kSeg: run_seg_tile<LPR, CH, BT>(g, tile, a); break;
                 case kZero: run_zero_tile<LPR, CH, BT>(g, tile, a); break;
                 default: run_chunk_tile<LPR, CH, BT>(g, tile, reinterpret_cast<float*>(s_raw), a); break;
@@ -892,8 +942,8 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             Group g{};
             g.log_w = lf::ilog2(b.width);
             const int fit = tile_slots(lpr) >> g.log_w;     // ELL rows whose slots fit the LDS tile
-            const bool staged = !is_multi[k] && fit >= sw;
-            g.type = staged ? kEll : kSeg;
+            const bool staged = fit >= sw;
+            g.type = staged ? (is_multi[k] ? kEllSeg : kEll) : kSeg;
             g.rows_per_tile = staged ? std::min(kTileRows, fit) : std::max(sw, fit);
             g.n_items = b.num_ell_rows;
             g.n_tiles = lf::ceil_div(g.n_items, g.rows_per_tile);
