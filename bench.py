@@ -78,14 +78,37 @@ def cpu_baseline(wl, B_host, feat, budget_s=20.0):
     t0 = time.perf_counter()
     out = A @ Bf
     dt = time.perf_counter() - t0
-    return {
+    res = {
         "value": round(2.0 * sub_nnz * feat / dt / 1e9, 3),
         "unit": "GFLOP/s",
         "cores": 1,
         "kind": "port",
         "sample": f"scipy csr_matrix(f32) @ dense(f32), first {take} of {rows} rows "
                   f"({sub_nnz} nnz), 1 run, {dt:.2f} s",
-    }, out, take
+    }
+    # the same sample through torch's threaded CPU CSR product, as a multi-core figure
+    try:
+        import warnings
+        import torch
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            At = torch.sparse_csr_tensor(torch.from_numpy(np.asarray(A.indptr, dtype=np.int64)),
+                                         torch.from_numpy(np.asarray(A.indices, dtype=np.int64)),
+                                         torch.from_numpy(A.data), size=A.shape)
+        Bt = torch.from_numpy(Bf)
+        At @ Bt                                             # warm-up (thread pool, first touch)
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            At @ Bt
+            times.append(time.perf_counter() - t0)
+        res["threaded"] = {"value": round(2.0 * sub_nnz * feat / float(np.median(times)) / 1e9, 3),
+                           "unit": "GFLOP/s", "cores": int(torch.get_num_threads()),
+                           "host_cpus": os.cpu_count(),
+                           "sample": "torch.sparse_csr_tensor(f32) @ dense(f32), same rows, median of 3"}
+    except Exception as exc:                                # a baseline only: report, do not fail the bench
+        res["threaded"] = {"value": None, "error": f"{type(exc).__name__}: {exc}"}
+    return res, out, take
 
 
 def bench_bsr(args):

@@ -42,11 +42,17 @@ constexpr int kWG = 256;            // threads per workgroup (4 wavefronts)
 #ifndef LF_UNROLL
 #define LF_UNROLL 8
 #endif
+#ifndef LF_TILE_MIN
+#define LF_TILE_MIN 512
+#endif
+#ifndef LF_EXTRA_LDS
+#define LF_EXTRA_LDS 0
+#endif
 // (col, val) pairs staged in LDS per tile: a fixed amount of work per sub-wave, so narrow
 // feature sizes (many sub-waves per workgroup) get larger tiles.  N = 128 -> 512 slots.
 constexpr int tile_slots(int lpr) {
     const int n = LF_TILE_SLOTS_PER_SUBWAVE * (kWG / lpr);
-    return n < 512 ? 512 : n;
+    return n < LF_TILE_MIN ? LF_TILE_MIN : n;
 }
 constexpr int kTileRows = 512;      // ELL rows per tile at most (<= tile_slots)
 #ifndef LF_COOP_SLOTS
@@ -1032,7 +1038,7 @@ int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t str
         a.B = d_B;
         a.C = d_C;
         a.partials = plan->d_partials;
-        ks.tiles<<<L.grid, kWG, 0, s>>>(a);
+        ks.tiles<<<L.grid, kWG, LF_EXTRA_LDS, s>>>(a);
         LF_HIP(hipGetLastError());
         if (L.n_heavy > 0) {
             const int sw = kWG / plan->lpr;
