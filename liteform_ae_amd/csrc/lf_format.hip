@@ -25,6 +25,7 @@ namespace {
 
 constexpr int kBlock = 256;          // rows per workgroup in the per-segment kernels
 constexpr int kSlotsPerThread = 4;   // slab slots written per thread in the scatter
+constexpr int kStatsGrid = 2048;     // workgroups per partition in the statistics pass at most
 constexpr int kLongSeg = 128;        // segments longer than this are walked by a whole wave
 // meta word of an ELL row: bits 0..10 valid slots (1..1024); bits 11..30 a count: on the
 // first ELL row of a source row's segment the number of ELL rows in the segment, on a
@@ -131,40 +132,44 @@ bucket_stats_kernel(SegView v, const int32_t* __restrict__ indices, const int32_
     __syncthreads();
 
     const int p = blockIdx.y;
-    const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    int start = 0, fill = 0, deg = 0;
-    if (r < v.rows) {
-        seg_range(v, r, p, start, fill);
-        deg = seg_deg ? seg_deg[(int64_t)p * v.rows + r] : fill;
-    }
-    uint32_t bit = 0;
-    if (deg > 0) {
-        int k, cost_rows;
-        width_class(deg, kmax, k, cost_rows);
-        bit = 1u << k;
-        atomicAdd(&s_stats[k * LF_STATS_FIELDS + 0], (unsigned long long)cost_rows);
-        atomicAdd(&s_stats[k * LF_STATS_FIELDS + 1], (unsigned long long)deg);
-        atomicAdd(&s_stats[k * LF_STATS_FIELDS + 2], 1ull);
-    }
-    if (colmask == nullptr) bit = 0;
-    const bool is_long = bit != 0 && fill > kLongSeg;
-    if (bit != 0 && !is_long) {
-        for (int i = 0; i < fill; ++i) {
-            const int c = indices[start + i];
-            if ((colmask[c] & bit) == 0) atomicOr(&colmask[c], bit);
-        }
-    }
-    unsigned long long pending = __ballot(is_long);
     const int lane = threadIdx.x & 63;
-    while (pending) {
-        const int src = __ffsll((long long)pending) - 1;
-        pending &= pending - 1;
-        const int s = __shfl(start, src);
-        const int f = __shfl(fill, src);
-        const uint32_t b = (uint32_t)__shfl((int)bit, src);
-        for (int i = lane; i < f; i += 64) {
-            const int c = indices[s + i];
-            if ((colmask[c] & b) == 0) atomicOr(&colmask[c], b);
+    // a workgroup walks several blocks of rows, so that the global counters below see a few
+    // thousand updates per launch and not one per 256 rows
+    for (int64_t base = (int64_t)blockIdx.x * kBlock; base < v.rows; base += (int64_t)gridDim.x * kBlock) {
+        const int64_t r = base + threadIdx.x;
+        int start = 0, fill = 0, deg = 0;
+        if (r < v.rows) {
+            seg_range(v, r, p, start, fill);
+            deg = seg_deg ? seg_deg[(int64_t)p * v.rows + r] : fill;
+        }
+        uint32_t bit = 0;
+        if (deg > 0) {
+            int k, cost_rows;
+            width_class(deg, kmax, k, cost_rows);
+            bit = 1u << k;
+            atomicAdd(&s_stats[k * LF_STATS_FIELDS + 0], (unsigned long long)cost_rows);
+            atomicAdd(&s_stats[k * LF_STATS_FIELDS + 1], (unsigned long long)deg);
+            atomicAdd(&s_stats[k * LF_STATS_FIELDS + 2], 1ull);
+        }
+        if (colmask == nullptr) bit = 0;
+        const bool is_long = bit != 0 && fill > kLongSeg;
+        if (bit != 0 && !is_long) {
+            for (int i = 0; i < fill; ++i) {
+                const int c = indices[start + i];
+                if ((colmask[c] & bit) == 0) atomicOr(&colmask[c], bit);
+            }
+        }
+        unsigned long long pending = __ballot(is_long);
+        while (pending) {
+            const int src = __ffsll((long long)pending) - 1;
+            pending &= pending - 1;
+            const int s = __shfl(start, src);
+            const int f = __shfl(fill, src);
+            const uint32_t b = (uint32_t)__shfl((int)bit, src);
+            for (int i = lane; i < f; i += 64) {
+                const int c = indices[s + i];
+                if ((colmask[c] & b) == 0) atomicOr(&colmask[c], b);
+            }
         }
     }
     __syncthreads();
@@ -267,12 +272,13 @@ hyb_scan_kernel(int32_t* __restrict__ blockcnt, int nblk, long long* __restrict_
 }
 
 // Writes, for every ELL row, its source row and meta word.  The in-block position comes
-// from one block-wide exclusive scan per bucket.
+// from per-wavefront counts per bucket (bit counts, or a shuffle scan where segments split)
+// combined through LDS with a single barrier.
 __global__ void __launch_bounds__(kBlock)
 hyb_rows_kernel(SegView v, const int32_t* __restrict__ seg_deg, const int32_t* __restrict__ wtab,
                 int nblk, const int32_t* __restrict__ blockoff, const long long* __restrict__ row_off,
                 int32_t* __restrict__ out_rows, int32_t* __restrict__ out_meta) {
-    __shared__ int s_wave[kBlock / 64];
+    __shared__ int s_cnt[kBlock / 64][LF_MAX_CLASSES + 1];
     const int p = blockIdx.y;
     const int32_t* w = wtab + p * kWtabStride;
     const int n = w[0];
@@ -290,21 +296,31 @@ hyb_rows_kernel(SegView v, const int32_t* __restrict__ seg_deg, const int32_t* _
             n_ell = (fill + width - 1) / width;
         }
     }
-    long long first = 0;      // flat ELL-row index of this segment's first ELL row
+    // ELL rows of the same bucket that precede this segment inside its wavefront.  Only the
+    // widest bucket splits segments; where every segment is one ELL row a bit count does it.
+    int in_wave = 0;
     for (int b = 0; b < n; ++b) {
-        const int x = mine == b ? n_ell : 0;
-        int incl = x;
-        for (int d = 1; d < 64; d <<= 1) {
-            const int y = __shfl_up(incl, d);
-            if (lane >= d) incl += y;
+        const unsigned long long members = __ballot(mine == b);
+        if (__ballot(mine == b && n_ell != 1) == 0) {
+            if (mine == b) in_wave = __popcll(members & ((1ull << lane) - 1ull));
+            if (lane == 0) s_cnt[wave][b] = __popcll(members);
+        } else {
+            const int x = mine == b ? n_ell : 0;
+            int incl = x;
+            for (int d = 1; d < 64; d <<= 1) {
+                const int y = __shfl_up(incl, d);
+                if (lane >= d) incl += y;
+            }
+            if (mine == b) in_wave = incl - x;
+            if (lane == 63) s_cnt[wave][b] = incl;
         }
-        if (lane == 63) s_wave[wave] = incl;
-        __syncthreads();
+    }
+    __syncthreads();
+    long long first = 0;      // flat ELL-row index of this segment's first ELL row
+    if (mine >= 0) {
         int wave_off = 0;
-        for (int wv = 0; wv < wave; ++wv) wave_off += s_wave[wv];
-        if (mine == b)
-            first = row_off[kbase + b] + blockoff[(int64_t)(kbase + b) * nblk + blockIdx.x] + wave_off + incl - x;
-        __syncthreads();
+        for (int wv = 0; wv < wave; ++wv) wave_off += s_cnt[wv][mine];
+        first = row_off[kbase + mine] + blockoff[(int64_t)(kbase + mine) * nblk + blockIdx.x] + wave_off + in_wave;
     }
     const bool is_long = n_ell > 8;
     if (n_ell > 0 && !is_long) {
@@ -349,34 +365,61 @@ hyb_scatter_kernel(const ScatterBucket* __restrict__ buckets, int nb, SegView v,
                    const int32_t* __restrict__ indices, const float* __restrict__ values,
                    const int32_t* __restrict__ rows, const int32_t* __restrict__ meta,
                    int32_t* __restrict__ out_cols, float* __restrict__ out_vals, float* __restrict__ out_mask) {
-    int lo = 0, hi = nb - 1;
-    while (lo < hi) {                      // last bucket whose block_start <= blockIdx.x
-        const int mid = (lo + hi + 1) >> 1;
-        if (buckets[mid].block_start <= (int)blockIdx.x) lo = mid; else hi = mid - 1;
+    // block_start ascends, so the bucket is (number of starts <= this workgroup) - 1; every
+    // wavefront counts them with one load per lane instead of a chain of dependent loads
+    const int lane = threadIdx.x & 63;
+    int k = -1;
+    for (int base = 0; base < nb; base += 64) {
+        const int i = base + lane;
+        const bool le = i < nb && buckets[i].block_start <= (int)blockIdx.x;
+        k += __popcll(__ballot(le));
     }
-    const ScatterBucket bk = buckets[lo];
+    const ScatterBucket bk = buckets[__builtin_amdgcn_readfirstlane(k)];
     const long long t0 = ((long long)(blockIdx.x - bk.block_start) * kBlock + threadIdx.x) * kSlotsPerThread;
     if (t0 >= bk.n_slots) return;
     const int wmask = (1 << bk.log_w) - 1;
     int32_t c[kSlotsPerThread];
     float x[kSlotsPerThread], m[kSlotsPerThread];
 #pragma unroll
-    for (int u = 0; u < kSlotsPerThread; ++u) {
-        const long long t = t0 + u;
-        c[u] = 0; x[u] = 0.f; m[u] = 0.f;
-        if (t < bk.n_slots) {
-            const long long e = bk.row_off + (t >> bk.log_w);
-            const int s = (int)(t & wmask);
-            const uint32_t mw = (uint32_t)meta[e];
-            const int len = (int)(mw & ((1u << kMetaLenBits) - 1));
-            if (s < len) {
-                int start, fill;
-                seg_range(v, rows[e], bk.part, start, fill);
-                const int idx = (mw & kMetaCont) ? (int)((mw & ~kMetaCont) >> kMetaLenBits) : 0;
-                const int at = start + (idx << bk.log_w) + s;
-                c[u] = indices[at];
-                x[u] = values ? values[at] : 1.0f;
-                m[u] = 1.0f;
+    for (int u = 0; u < kSlotsPerThread; ++u) { c[u] = 0; x[u] = 0.f; m[u] = 0.f; }
+    if (bk.log_w >= 2) {
+        // the thread's slots lie in one ELL row: one look-up of the row, its segment and meta
+        const long long e = bk.row_off + (t0 >> bk.log_w);
+        const int s0 = (int)(t0 & wmask);
+        const uint32_t mw = (uint32_t)meta[e];
+        const int len = (int)(mw & ((1u << kMetaLenBits) - 1));
+        if (s0 < len) {
+            int start, fill;
+            seg_range(v, rows[e], bk.part, start, fill);
+            const int idx = (mw & kMetaCont) ? (int)((mw & ~kMetaCont) >> kMetaLenBits) : 0;
+            const int at = start + (idx << bk.log_w) + s0;
+#pragma unroll
+            for (int u = 0; u < kSlotsPerThread; ++u) {
+                if (s0 + u < len) {
+                    c[u] = indices[at + u];
+                    x[u] = values ? values[at + u] : 1.0f;
+                    m[u] = 1.0f;
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < kSlotsPerThread; ++u) {
+            const long long t = t0 + u;
+            if (t < bk.n_slots) {
+                const long long e = bk.row_off + (t >> bk.log_w);
+                const int s = (int)(t & wmask);
+                const uint32_t mw = (uint32_t)meta[e];
+                const int len = (int)(mw & ((1u << kMetaLenBits) - 1));
+                if (s < len) {
+                    int start, fill;
+                    seg_range(v, rows[e], bk.part, start, fill);
+                    const int idx = (mw & kMetaCont) ? (int)((mw & ~kMetaCont) >> kMetaLenBits) : 0;
+                    const int at = start + (idx << bk.log_w) + s;
+                    c[u] = indices[at];
+                    x[u] = values ? values[at] : 1.0f;
+                    m[u] = 1.0f;
+                }
             }
         }
     }
@@ -546,7 +589,7 @@ int lf_bucket_stats(const int32_t* d_indptr, const int32_t* d_indices, const int
             LF_HIP(hipGetLastError());
         }
         SegView v{d_indptr, bnd, num_rows, num_parts};
-        bucket_stats_kernel<<<dim3(nblk, num_parts), kBlock, 0, s>>>(v, d_indices, d_seg_deg,
+        bucket_stats_kernel<<<dim3(std::min(nblk, kStatsGrid), num_parts), kBlock, 0, s>>>(v, d_indices, d_seg_deg,
                                                                      lf::ilog2(width_limit),
                                                                      h_colhist ? colmask : nullptr, stats);
         LF_HIP(hipGetLastError());
