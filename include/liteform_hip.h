@@ -93,6 +93,14 @@ int lf_coo_degrees(const int32_t* d_coo_row, const int32_t* d_coo_col, int64_t n
                    int64_t num_rows, int64_t num_cols, int32_t num_parts,
                    int32_t* d_seg_deg, lf_stream_t stream);
 
+/* Row-length statistics of a CSR matrix, the integer part of MTX.matrix_features
+ * (format_matrix_market.py:153-202): h_out = {min, max, sum, sum of squares} of the row
+ * lengths indptr[r+1] - indptr[r] (exact integers; mean and standard deviation follow on
+ * the host).  num_rows == 0 gives {0, 0, 0, 0}.  d_scratch: 32 bytes of device memory.
+ * Synchronises the stream. */
+int lf_row_features(const int32_t* d_indptr, int64_t num_rows, void* d_scratch,
+                    int64_t* h_out /* [4] */, lf_stream_t stream);
+
 /* ------------------------------------------------------------------------------------
  * Bucket-width search on the host (no GPU work).  Replaces modify_single_row_buckets,
  * get_bucket_config, modify_bucket_widths, move_largest_bucket, move_width_one_bucket and

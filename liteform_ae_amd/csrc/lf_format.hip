@@ -106,6 +106,42 @@ __global__ void coo_degree_kernel(const int32_t* __restrict__ row, const int32_t
     }
 }
 
+// out = {min, max, sum, sum of squares} of the row lengths; out[0] starts at ~0, the rest at 0
+__global__ void __launch_bounds__(kBlock)
+row_features_kernel(const int32_t* __restrict__ indptr, int64_t rows, unsigned long long* __restrict__ out) {
+    __shared__ unsigned long long s_red[4][kBlock / 64];
+    unsigned long long lo = ~0ull, hi = 0, sum = 0, sq = 0;
+    for (int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x; r < rows; r += (int64_t)gridDim.x * kBlock) {
+        const unsigned long long d = (unsigned long long)(indptr[r + 1] - indptr[r]);
+        lo = d < lo ? d : lo;
+        hi = d > hi ? d : hi;
+        sum += d;
+        sq += d * d;
+    }
+    for (int d = 32; d > 0; d >>= 1) {
+        const unsigned long long l2 = __shfl_xor(lo, d), h2 = __shfl_xor(hi, d);
+        lo = l2 < lo ? l2 : lo;
+        hi = h2 > hi ? h2 : hi;
+        sum += __shfl_xor(sum, d);
+        sq += __shfl_xor(sq, d);
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) { s_red[0][wave] = lo; s_red[1][wave] = hi; s_red[2][wave] = sum; s_red[3][wave] = sq; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kBlock / 64; ++w) {
+            lo = s_red[0][w] < lo ? s_red[0][w] : lo;
+            hi = s_red[1][w] > hi ? s_red[1][w] : hi;
+            sum += s_red[2][w];
+            sq += s_red[3][w];
+        }
+        atomicMin(&out[0], lo);
+        atomicMax(&out[1], hi);
+        atomicAdd(&out[2], sum);
+        atomicAdd(&out[3], sq);
+    }
+}
+
 // Initial width class of a segment of `deg` entries: width = min(next_pow2(deg), limit),
 // cost-model rows = max(1, next_pow2(deg) / limit)            (format_algos.py:875-882)
 __device__ __forceinline__ void width_class(int deg, int kmax, int& k, int& cost_rows) {
@@ -646,6 +682,26 @@ int lf_bucket_stats(const int32_t* d_indptr, const int32_t* d_indices, const int
     }
     LF_HIP(hipMemcpyAsync(h_stats, stats, stats_bytes, hipMemcpyDeviceToHost, s));
     if (h_colhist) LF_HIP(hipMemcpyAsync(h_colhist, hist, hist_bytes, hipMemcpyDeviceToHost, s));
+    LF_HIP(hipStreamSynchronize(s));
+    return LF_OK;
+}
+
+int lf_row_features(const int32_t* d_indptr, int64_t num_rows, void* d_scratch, int64_t* h_out,
+                    lf_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    LF_REQUIRE(h_out, LF_ERR_INVALID, "h_out is null");
+    LF_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31), LF_ERR_INVALID, "bad num_rows");
+    h_out[0] = h_out[1] = h_out[2] = h_out[3] = 0;
+    if (num_rows == 0) return LF_OK;
+    LF_REQUIRE(d_indptr && d_scratch, LF_ERR_INVALID, "null argument");
+    LF_REQUIRE((uintptr_t)d_scratch % 8 == 0, LF_ERR_INVALID, "scratch must be 8-byte aligned");
+    unsigned long long* acc = (unsigned long long*)d_scratch;
+    LF_HIP(fill_u32(acc, 2, 0xFFFFFFFFu, s));
+    LF_HIP(fill_u32(acc + 1, 6, 0u, s));
+    const int grid = (int)std::min<int64_t>((num_rows + kBlock - 1) / kBlock, 1024);
+    row_features_kernel<<<grid, kBlock, 0, s>>>(d_indptr, num_rows, acc);
+    LF_HIP(hipGetLastError());
+    LF_HIP(hipMemcpyAsync(h_out, acc, 32, hipMemcpyDeviceToHost, s));
     LF_HIP(hipStreamSynchronize(s));
     return LF_OK;
 }

@@ -35,7 +35,7 @@ from .format_matrix_market import MTX, Bucket  # noqa: F401  (re-exported like t
 __all__ = ["build_hyb_format", "bench_hyb_with_config", "search_bucket_config",
            "CostModelSettings", "bench_bsrmm", "bench_naive", "spmm_bsr",
            "build_hyb_format_device", "HybFormat", "HybSpMM", "spmm_hyb", "spmm_csr",
-           "guess_num_partitions", "choose_num_partitions"]
+           "guess_num_partitions", "choose_num_partitions", "matrix_features_device"]
 
 WIDTH_LIMIT = 1024   # format_algos.py:821
 
@@ -581,6 +581,40 @@ def bench_naive(g, x, y_ndarray, feat_size=128, coarsening_factor=2, check_corre
 
 
 # --------------------------------------------------------------------------- partition count
+def matrix_features_device(g) -> dict:
+    """``MTX.matrix_features`` (format_matrix_market.py:153-202) with the pass over the
+    row pointer done on the GPU: the kernel returns min, max, sum and sum of squares of the
+    row lengths as exact integers; mean, standard deviation and the densities follow from
+    them in float64 (the standard deviation as sqrt(E[d^2] - E[d]^2), which agrees with
+    numpy's two-pass value to ~1e-12 relative for these integer inputs)."""
+    torch = _torch()
+    lib = _lib.load()
+    dev = _device_csr(g)
+    out = np.zeros(4, dtype=np.int64)
+    scratch = torch.empty(4, dtype=torch.int64, device="cuda")
+    _lib.check(lib.lf_row_features(_lib.ptr(dev.indptr), dev.num_rows, _lib.ptr(scratch),
+                                   _lib.np_ptr(out, C.c_int64), _stream()))
+    rows, cols = dev.num_rows, dev.num_cols
+    lo, hi, total, squares = (int(x) for x in out)
+    mean = total / rows if rows else 0.0
+    var = max(0.0, squares / rows - mean * mean) if rows else 0.0
+    std = float(np.sqrt(var))
+    return {
+        "name": getattr(g, "name", None),
+        "num_rows": rows,
+        "num_cols": cols,
+        "nnz": dev.coo_nnz,                      # stored COO entries, as the reference reports
+        "avg_nnz_per_row": mean,
+        "min_nnz_per_row": lo,
+        "max_nnz_per_row": hi,
+        "std_dev_nnz_per_row": std,
+        "avg_nnz_density_per_row": mean / cols,
+        "min_nnz_density_per_row": lo / cols,
+        "max_nnz_density_per_row": hi / cols,
+        "std_dev_nnz_density_per_row": std / cols,
+    }
+
+
 MALL_BYTES = 256 << 20        # MI355X memory-side cache (Infinity Cache)
 
 

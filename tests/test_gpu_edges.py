@@ -131,3 +131,22 @@ def test_graph_replay_matches_eager(fa, torch):
         torch.cuda.synchronize()
         assert torch.equal(out, plan.run(B))
         plan.close()
+
+
+def test_matrix_features_on_device(fa, torch):
+    """Integer fields exact, float fields to 1e-9 relative against the host routine
+    (numpy's two-pass standard deviation against sqrt(E[d^2] - E[d]^2) on exact sums)."""
+    rng = np.random.default_rng(11)
+    g = skewed_matrix(rng, 5000, 3000, mean_deg=7.0, heavy_rows=3, heavy_len=2500)
+    # duplicated COO entries: "nnz" counts stored entries, row lengths come from the CSR
+    row = np.concatenate([g.coo_mtx.row, g.coo_mtx.row[:100]])
+    col = np.concatenate([g.coo_mtx.col, g.coo_mtx.col[:100]])
+    for m in (g, MTX.from_coo(row, col, g.coo_mtx.shape), mtx_from_rows([[], [1], []], (3, 4))):
+        want = m.matrix_features()
+        got = fa.matrix_features_device(m)
+        assert list(got) == list(want)
+        for key in ("name", "num_rows", "num_cols", "nnz", "min_nnz_per_row", "max_nnz_per_row"):
+            assert got[key] == want[key], key
+        for key in want:
+            if key.startswith(("avg", "std", "min_nnz_density", "max_nnz_density")):
+                assert got[key] == pytest.approx(want[key], rel=1e-9, abs=1e-15), key
