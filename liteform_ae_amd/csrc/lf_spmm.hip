@@ -297,7 +297,11 @@ __device__ __forceinline__ void ell_tile_wide(const int2* s_pairs, const int2* s
         const int c0 = rp[0].x;
         Acc<CH, VEC> acc;
         acc.clear();
-        for (int j = 0; j < len; j += kUnroll) {
+        // Whole groups of kUnroll slots, then a tail of kUnroll or kUnroll / 2 gathers.  The
+        // short tail saves padding gathers (a 27-slot stencil row: 28 instead of 32); with
+        // many rows per wavefront (small N) the extra branch costs more than it saves.
+        constexpr bool kShortTail = LPR >= 32;
+        auto group = [&](int j) {                     // kUnroll slots from j, padding redirected
             int c[kUnroll];
             float v[kUnroll];
 #pragma unroll
@@ -307,6 +311,26 @@ __device__ __forceinline__ void ell_tile_wide(const int2* s_pairs, const int2* s
                 v[u] = __int_as_float(cv.y);
             }
             gather_fma<kUnroll, LPR, CH, BT>(a.B, ln, c, v, acc);
+        };
+        if constexpr (kShortTail) {
+            int j = 0;
+            for (; j + kUnroll <= len; j += kUnroll) group(j);
+            if (len > j && len - j <= kUnroll / 2) {
+                constexpr int H = kUnroll / 2;
+                int c[H];
+                float v[H];
+#pragma unroll
+                for (int u = 0; u < H; ++u) {
+                    const int2 cv = rp[j + u];
+                    c[u] = j + u < len ? cv.x : c0;
+                    v[u] = __int_as_float(cv.y);
+                }
+                gather_fma<H, LPR, CH, BT>(a.B, ln, c, v, acc);
+            } else if (len > j) {
+                group(j);
+            }
+        } else {
+            for (int j = 0; j < len; j += kUnroll) group(j);
         }
         store_row<LPR, CH, VEC>(a.C, rm.x, ln, acc, a.accumulate);
     }
