@@ -45,9 +45,6 @@ constexpr int kWG = 256;            // threads per workgroup (4 wavefronts)
 #ifndef LF_TILE_MIN
 #define LF_TILE_MIN 512
 #endif
-#ifndef LF_EXTRA_LDS
-#define LF_EXTRA_LDS 0
-#endif
 // (col, val) pairs staged in LDS per tile: a fixed amount of work per sub-wave, so narrow
 // feature sizes (many sub-waves per workgroup) get larger tiles.  N = 128 -> 512 slots.
 constexpr int tile_slots(int lpr) {
@@ -64,6 +61,7 @@ constexpr int kTileRows = 512;      // ELL rows per tile at most (<= tile_slots)
 constexpr int kCoopSlots = LF_COOP_SLOTS;    // a source row with more slab slots is reduced by a whole workgroup
 constexpr int kChunkSlots = LF_CHUNK_SLOTS;  // ... in chunks of this many slots (a whole number of ELL rows)
 constexpr int kXcds = 8;
+constexpr int kPartBytesMax = 16384;   // LDS for per-ELL-row sums of a balanced segment tile at most
 constexpr int kUnroll = LF_UNROLL;  // B-row gathers in flight per sub-wave
 constexpr uint32_t kMetaLenMask = 0x7FFu;
 constexpr int kMetaLenBits = 11;
@@ -90,7 +88,7 @@ struct Group {
     int type;
     int log_w;
     int rows_per_tile;
-    int pad_;
+    int balanced;                 // kEllSeg: per-ELL-row sums through LDS (needs rows_per_tile * N floats)
     long long n_items;            // ELL rows / rows to clear / chunks
     long long n_tiles;
     const int32_t* rows;          // kEll, kSeg: source rows; kZero: rows to clear
@@ -342,12 +340,19 @@ __device__ __forceinline__ void ell_tile_wide(const int2* s_pairs, const int2* s
 // global memory.  Continuation rows and rows that take the cooperative path are skipped.
 template <int LPR, int CH, typename BT>
 __device__ __forceinline__ void ell_tile_segments(const Group& g, long long e0, const int2* s_pairs,
-                                                  const int2* s_rm, int n, const LaunchArgs& a, int sw, int sl) {
+                                                  const int2* s_rm, int n, const LaunchArgs& a, int* s_next,
+                                                  int sl) {
     constexpr int VEC = Dense<BT>::kVec;
-    constexpr int SW = kWG / LPR;
     const Lane<LPR, CH, VEC> ln(sl, a.feat);
     const int log_w = g.log_w;
-    for (int r = sw; r < n; r += SW) {
+    // Segments differ in length and continuation rows carry no work, so the sub-waves take
+    // the tile's ELL rows from a shared counter as they become free instead of by a fixed
+    // stride.  Which sub-wave sums a row does not change the order of its additions.
+    for (;;) {
+        int r = 0;
+        if (sl == 0) r = atomicAdd(s_next, 1);
+        r = __shfl(r, 0, LPR);
+        if (r >= n) break;
         const int2 rm = s_rm[r];
         if (rm.y < 0) continue;                                  // continuation row
         const int seg = (int)((uint32_t)rm.y >> kMetaLenBits);
@@ -381,9 +386,90 @@ __device__ __forceinline__ void ell_tile_segments(const Group& g, long long e0, 
     }
 }
 
+// The same bucket with the work spread evenly: every ELL row of the tile is summed by the
+// sub-wave it falls to, a row that is only part of a segment leaves its sum in LDS, and after
+// a barrier the first ELL row of each segment adds the sums of its rows in order.  With the
+// variant above a tile of a folded configuration offers fewer segments than sub-waves at
+// small N (about 20 for 32 at N = 32), and the lanes in flight bound the gather rate.
+// Rows that continue a segment begun in an earlier tile are summed by that tile, as above.
+template <int LPR, int CH, typename BT>
+__device__ __forceinline__ void ell_tile_segments_balanced(const Group& g, long long e0, const int2* s_pairs,
+                                                           const int2* s_rm, int n, const LaunchArgs& a,
+                                                           float* s_part, int sw, int sl) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int SW = kWG / LPR;
+    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const int log_w = g.log_w;
+    for (int r = sw; r < n; r += SW) {
+        const int2 rm = s_rm[r];
+        const bool cont = rm.y < 0;
+        const int head = cont ? r - (int)(((uint32_t)rm.y & 0x7FFFFFFFu) >> kMetaLenBits) : r;
+        if (head < 0) continue;                                  // belongs to the previous tile's last segment
+        const int seg = (int)((uint32_t)s_rm[head].y >> kMetaLenBits);
+        if (((long long)seg << log_w) > kCoopSlots) continue;   // reduced by a whole workgroup
+        const int len = rm.y & kMetaLenMask;
+        const int2* rp = s_pairs + (r << log_w);
+        const int c0 = rp[0].x;
+        Acc<CH, VEC> acc;
+        acc.clear();
+        for (int j = 0; j < len; j += kUnroll) {
+            int c[kUnroll];
+            float v[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const int2 cv = rp[j + u];
+                c[u] = j + u < len ? cv.x : c0;
+                v[u] = __int_as_float(cv.y);
+            }
+            gather_fma<kUnroll, LPR, CH, BT>(a.B, ln, c, v, acc);
+        }
+        if (seg == 1) {
+            store_row<LPR, CH, VEC>(a.C, rm.x, ln, acc, a.accumulate);
+        } else {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                if (!ln.on[c]) continue;
+                float* dst = s_part + r * a.feat + ln.f[c];
+#pragma unroll
+                for (int i = 0; i < VEC; i += 4)
+                    *reinterpret_cast<float4*>(dst + i) =
+                        make_float4(acc.v[c][i], acc.v[c][i + 1], acc.v[c][i + 2], acc.v[c][i + 3]);
+            }
+        }
+    }
+    __syncthreads();
+    for (int r = sw; r < n; r += SW) {
+        const int2 rm = s_rm[r];
+        if (rm.y < 0) continue;
+        const int seg = (int)((uint32_t)rm.y >> kMetaLenBits);
+        if (seg == 1 || ((long long)seg << log_w) > kCoopSlots) continue;
+        Acc<CH, VEC> acc;
+        acc.clear();
+        const int inside = min(seg, n - r);
+        for (int k = 0; k < inside; ++k) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                if (!ln.on[c]) continue;
+                const float* src = s_part + (r + k) * a.feat + ln.f[c];
+#pragma unroll
+                for (int i = 0; i < VEC; i += 4) {
+                    const float4 x = *reinterpret_cast<const float4*>(src + i);
+                    acc.v[c][i] += x.x; acc.v[c][i + 1] += x.y; acc.v[c][i + 2] += x.z; acc.v[c][i + 3] += x.w;
+                }
+            }
+        }
+        if (inside < seg) {                                      // the segment runs past the tile: stream the rest
+            const int total = ((seg - 1) << log_w) + (g.meta[e0 + r + seg - 1] & kMetaLenMask);
+            const int staged = inside << log_w;
+            stream_slots<LPR, CH, BT>(g.cols, g.vals, ((e0 + r) << log_w) + staged, total - staged, a.B, ln, acc);
+        }
+        store_row<LPR, CH, VEC>(a.C, rm.x, ln, acc, a.accumulate);
+    }
+}
+
 template <int LPR, int CH, typename BT>
 __device__ __forceinline__ void run_ell_tile(const Group& g, long long tile, int2* s_pairs, int2* s_rm,
-                                             const LaunchArgs& a) {
+                                             int* s_next, float* s_part, const LaunchArgs& a) {
     const int tid = threadIdx.x;
     const long long e0 = tile * g.rows_per_tile;
     const int n = (int)min((long long)g.rows_per_tile, g.n_items - e0);
@@ -403,10 +489,12 @@ __device__ __forceinline__ void run_ell_tile(const Group& g, long long tile, int
         }
     }
     for (int i = tid; i < n; i += kWG) s_rm[i] = make_int2(g.rows[e0 + i], g.meta[e0 + i]);
+    if (tid == 0) *s_next = 0;
     __syncthreads();
     const int sw = tid / LPR, sl = tid % LPR;
     if (g.type == kEllSeg) {
-        ell_tile_segments<LPR, CH, BT>(g, e0, s_pairs, s_rm, n, a, sw, sl);
+        if (g.balanced) ell_tile_segments_balanced<LPR, CH, BT>(g, e0, s_pairs, s_rm, n, a, s_part, sw, sl);
+        else ell_tile_segments<LPR, CH, BT>(g, e0, s_pairs, s_rm, n, a, s_next, sl);
         return;
     }
     switch (g.log_w) {
@@ -528,6 +616,8 @@ spmm_partition_kernel(LaunchArgs a) {
     __shared__ __align__(16) char s_raw[kStageBytes > kReduceBytes ? kStageBytes : kReduceBytes];
     int2* s_pairs = reinterpret_cast<int2*>(s_raw);
     int2* s_rm = s_pairs + kTileSlots;
+    __shared__ int s_next;                     // next ELL row of a tile whose rows are taken dynamically
+    extern __shared__ __align__(16) float s_dyn[];   // per-ELL-row sums of a balanced segment tile
 
     const int xcd = blockIdx.x % kXcds;
     long long v = blockIdx.x / kXcds;          // position in this XCD's tile list
@@ -539,7 +629,7 @@ spmm_partition_kernel(LaunchArgs a) {
             const long long tile = lo + v;
             switch (g.type) {
                 case kEll:
-                case kEllSeg: run_ell_tile<LPR, CH, BT>(g, tile, s_pairs, s_rm, a); break;
+                case kEllSeg: run_ell_tile<LPR, CH, BT>(g, tile, s_pairs, s_rm, &s_next, s_dyn, a); break;
                 case kSeg: run_seg_tile<LPR, CH, BT>(g, tile, a); break;
                 case kZero: run_zero_tile<LPR, CH, BT>(g, tile, a); break;
                 default: run_chunk_tile<LPR, CH, BT>(g, tile, reinterpret_cast<float*>(s_raw), a); break;
@@ -693,6 +783,7 @@ struct lf_spmm_plan {
     int device = 0, num_cus = 0, grid = 0;
     struct Launch {
         int group_begin = 0, n_groups = 0, grid = 0;
+        int dyn_lds = 0;             // bytes of dynamic LDS (balanced segment tiles)
         long long tiles = 0;
         int heavy_begin = 0, n_heavy = 0;
     };
@@ -975,6 +1066,13 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             const bool staged = fit >= sw;
             g.type = staged ? (is_multi[k] ? kEllSeg : kEll) : kSeg;
             g.rows_per_tile = staged ? std::min(kTileRows, fit) : std::max(sw, fit);
+            if (g.type == kEllSeg) {
+                const long long part_bytes = (long long)g.rows_per_tile * feat_size * 4;
+                if (part_bytes <= kPartBytesMax) {
+                    g.balanced = 1;
+                    L.dyn_lds = std::max(L.dyn_lds, (int)part_bytes);
+                }
+            }
             g.n_items = b.num_ell_rows;
             g.n_tiles = lf::ceil_div(g.n_items, g.rows_per_tile);
             g.rows = b.d_rows;
@@ -1015,9 +1113,13 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     KernelSet ks;
     LF_TRY(select_kernels(lpr, ch, b_dtype, &ks));
     int occ = 0;
-    LF_TRY_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, ks.tiles, kWG, 0));
+    int dyn_lds = 0;
     plan->grid = 0;
-    for (const auto& L : plan->launches) plan->grid = std::max(plan->grid, L.grid);
+    for (const auto& L : plan->launches) {
+        plan->grid = std::max(plan->grid, L.grid);
+        dyn_lds = std::max(dyn_lds, L.dyn_lds);
+    }
+    LF_TRY_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, ks.tiles, kWG, dyn_lds));
 
     plan->info[0] = total_tiles;
     plan->info[1] = plan->grid;
@@ -1025,7 +1127,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     {
         hipFuncAttributes fa;
         LF_TRY_HIP(hipFuncGetAttributes(&fa, reinterpret_cast<const void*>(ks.tiles)));
-        plan->info[3] = (int64_t)fa.sharedSizeBytes;
+        plan->info[3] = (int64_t)fa.sharedSizeBytes + dyn_lds;
     }
     plan->info[4] = n_heavy_total;
     plan->info[5] = n_partials;
@@ -1062,7 +1164,7 @@ int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t str
         a.B = d_B;
         a.C = d_C;
         a.partials = plan->d_partials;
-        ks.tiles<<<L.grid, kWG, LF_EXTRA_LDS, s>>>(a);
+        ks.tiles<<<L.grid, kWG, L.dyn_lds, s>>>(a);
         LF_HIP(hipGetLastError());
         if (L.n_heavy > 0) {
             const int sw = kWG / plan->lpr;

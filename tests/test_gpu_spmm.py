@@ -80,6 +80,23 @@ def test_every_width_path(fa, torch, widths):
     check(fa, torch, g, widths, 128)
 
 
+@pytest.mark.parametrize("feat,b_dtype", [(32, "f32"), (64, "f32"), (128, "f32"), (256, "f32"), (64, "bf16"),
+                                          (256, "bf16")])
+def test_folded_configurations_split_rows_over_ell_rows(fa, torch, feat, b_dtype):
+    """Widest bucket narrower than most rows: segments of 2..8 ELL rows (many cross a tile
+    boundary), summed row by row through LDS where the tile's partial sums fit."""
+    rng = np.random.default_rng(500 + feat)
+    g = skewed_matrix(rng, 2500, 3000, mean_deg=40, heavy_rows=3, heavy_len=2000)
+    plain = fa.HybSpMM(fa.build_hyb_format_device(g, [[1024]]), feat, b_dtype)
+    static_lds = plain.info["lds_bytes"]
+    plain.close()
+    for widths in ([[8]], [[16]], [[32]], [[1, 2, 4, 8, 16, 32]], [[64]], [[4, 16], [2, 32]]):
+        _, info = check(fa, torch, g, widths, feat, b_dtype, seed=feat)
+        rows_per_tile = max(512, 64 * 256 // (feat // (8 if b_dtype == "bf16" else 4))) // widths[0][-1]
+        if rows_per_tile * feat * 4 <= 16384 and len(widths) == 1:
+            assert info["lds_bytes"] > static_lds, (widths, info)
+
+
 @pytest.mark.parametrize("feat,b_dtype", [(32, "f32"), (128, "f32"), (512, "bf16")])
 def test_very_long_rows_are_split_into_chunks(fa, torch, feat, b_dtype):
     rng = np.random.default_rng(77)
