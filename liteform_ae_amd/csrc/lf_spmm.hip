@@ -281,6 +281,23 @@ __device__ __forceinline__ void ell_tile_narrow(const int2* s_pairs, const int2*
     }
 }
 
+// U staged slots of an ELL row from position j; slots at or past `len` are padding and are
+// redirected to the row's first column (their value is 0).
+template <int U, int LPR, int CH, typename BT>
+__device__ __forceinline__ void staged_group(const int2* rp, int j, int len, int c0, const void* B,
+                                             const Lane<LPR, CH, Dense<BT>::kVec>& ln,
+                                             Acc<CH, Dense<BT>::kVec>& acc) {
+    int c[U];
+    float v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int2 cv = rp[j + u];
+        c[u] = j + u < len ? cv.x : c0;
+        v[u] = __int_as_float(cv.y);
+    }
+    gather_fma<U, LPR, CH, BT>(B, ln, c, v, acc);
+}
+
 // Bucket with W >= kUnroll (a multiple of it) staged in LDS: one ELL row per sub-wave at a time.
 template <int LPR, int CH, typename BT>
 __device__ __forceinline__ void ell_tile_wide(const int2* s_pairs, const int2* s_rm, int n, int log_w,
@@ -299,36 +316,13 @@ __device__ __forceinline__ void ell_tile_wide(const int2* s_pairs, const int2* s
         // short tail saves padding gathers (a 27-slot stencil row: 28 instead of 32); with
         // many rows per wavefront (small N) the extra branch costs more than it saves.
         constexpr bool kShortTail = LPR >= 32;
-        auto group = [&](int j) {                     // kUnroll slots from j, padding redirected
-            int c[kUnroll];
-            float v[kUnroll];
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                const int2 cv = rp[j + u];
-                c[u] = j + u < len ? cv.x : c0;
-                v[u] = __int_as_float(cv.y);
-            }
-            gather_fma<kUnroll, LPR, CH, BT>(a.B, ln, c, v, acc);
-        };
         if constexpr (kShortTail) {
             int j = 0;
-            for (; j + kUnroll <= len; j += kUnroll) group(j);
-            if (len > j && len - j <= kUnroll / 2) {
-                constexpr int H = kUnroll / 2;
-                int c[H];
-                float v[H];
-#pragma unroll
-                for (int u = 0; u < H; ++u) {
-                    const int2 cv = rp[j + u];
-                    c[u] = j + u < len ? cv.x : c0;
-                    v[u] = __int_as_float(cv.y);
-                }
-                gather_fma<H, LPR, CH, BT>(a.B, ln, c, v, acc);
-            } else if (len > j) {
-                group(j);
-            }
+            for (; j + kUnroll <= len; j += kUnroll) staged_group<kUnroll, LPR, CH, BT>(rp, j, len, c0, a.B, ln, acc);
+            if (len > j && len - j <= kUnroll / 2) staged_group<kUnroll / 2, LPR, CH, BT>(rp, j, len, c0, a.B, ln, acc);
+            else if (len > j) staged_group<kUnroll, LPR, CH, BT>(rp, j, len, c0, a.B, ln, acc);
         } else {
-            for (int j = 0; j < len; j += kUnroll) group(j);
+            for (int j = 0; j < len; j += kUnroll) staged_group<kUnroll, LPR, CH, BT>(rp, j, len, c0, a.B, ln, acc);
         }
         store_row<LPR, CH, VEC>(a.C, rm.x, ln, acc, a.accumulate);
     }
