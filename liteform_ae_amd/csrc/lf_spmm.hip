@@ -712,26 +712,54 @@ __global__ void derive_meta_kernel(const int32_t* __restrict__ rows, const float
 // has rows spanning several ELL rows"); the second run fills the tables, taking ranges with
 // the same counters.  Table order depends on scheduling, results do not: every row's
 // partials are private and are summed in chunk order.
-__global__ void plan_chunks_kernel(const int32_t* __restrict__ rows, const int32_t* __restrict__ meta,
-                                   long long n_rows, int log_w, int* __restrict__ counters,
-                                   Chunk* __restrict__ chunks, HeavyRow* __restrict__ heavy,
-                                   int partial_base, int heavy_base) {
+__global__ void __launch_bounds__(256)
+plan_chunks_kernel(const int32_t* __restrict__ rows, const int32_t* __restrict__ meta,
+                   long long n_rows, int log_w, int* __restrict__ counters,
+                   Chunk* __restrict__ chunks, HeavyRow* __restrict__ heavy,
+                   int partial_base, int heavy_base) {
     const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n_rows) return;
-    const int m = meta[e];
-    if (m < 0) { counters[3] = 1; return; }
-    const int seg = (int)((uint32_t)m >> kMetaLenBits);
-    if (seg > 1) counters[3] = 1;
-    if (((long long)seg << log_w) <= kCoopSlots) return;
+    const int lane = threadIdx.x & 63;
+    int seg = 0, n_chunks = 0;
+    bool split = false;
     const int rows_per_chunk = max(1, kChunkSlots >> log_w);
-    const int n_chunks = (seg + rows_per_chunk - 1) / rows_per_chunk;
-    const int c0 = atomicAdd(&counters[0], n_chunks);
-    int h = 0, p0 = 0;
-    if (n_chunks > 1) {
-        h = atomicAdd(&counters[1], 1);
-        p0 = atomicAdd(&counters[2], n_chunks);
+    if (e < n_rows) {
+        const int m = meta[e];
+        if (m < 0) {
+            split = true;
+        } else {
+            seg = (int)((uint32_t)m >> kMetaLenBits);
+            split = seg > 1;
+            if (((long long)seg << log_w) > kCoopSlots) n_chunks = (seg + rows_per_chunk - 1) / rows_per_chunk;
+        }
     }
-    if (chunks == nullptr) return;
+    if (__ballot(split) != 0 && lane == 0) counters[3] = 1;
+    // ranges of the tables: one atomic per counter and wavefront (a matrix of long rows has
+    // a cooperative row in every lane)
+    const bool several = n_chunks > 1;
+    const int part = several ? n_chunks : 0;
+    int incl_c = n_chunks, incl_p = part;
+    for (int d = 1; d < 64; d <<= 1) {
+        const int yc = __shfl_up(incl_c, d), yp = __shfl_up(incl_p, d);
+        if (lane >= d) { incl_c += yc; incl_p += yp; }
+    }
+    const int tot_c = __shfl(incl_c, 63), tot_p = __shfl(incl_p, 63);
+    if (tot_c == 0) return;
+    const unsigned long long votes = __ballot(several);
+    int base_c = 0, base_h = 0, base_p = 0;
+    if (lane == 0) {
+        base_c = atomicAdd(&counters[0], tot_c);
+        if (votes) {
+            base_h = atomicAdd(&counters[1], __popcll(votes));
+            base_p = atomicAdd(&counters[2], tot_p);
+        }
+    }
+    base_c = __shfl(base_c, 0);
+    base_h = __shfl(base_h, 0);
+    base_p = __shfl(base_p, 0);
+    if (chunks == nullptr || n_chunks == 0) return;
+    const int c0 = base_c + incl_c - n_chunks;
+    const int h = base_h + __popcll(votes & ((1ull << lane) - 1ull));
+    const int p0 = base_p + incl_p - part;
     const long long total = ((long long)(seg - 1) << log_w) + (meta[e + seg - 1] & kMetaLenMask);
     const int row = rows[e];
     for (int i = 0; i < n_chunks; ++i) {
@@ -740,12 +768,12 @@ __global__ void plan_chunks_kernel(const int32_t* __restrict__ rows, const int32
         Chunk ck;
         ck.slot_begin = (e << log_w) + lo;
         ck.n_slots = (int)(hi - lo);
-        ck.partial = n_chunks > 1 ? partial_base + p0 + i : -1;
+        ck.partial = several ? partial_base + p0 + i : -1;
         ck.row = row;
         ck.pad_ = 0;
         chunks[c0 + i] = ck;
     }
-    if (n_chunks > 1) heavy[heavy_base + h] = HeavyRow{row, partial_base + p0, n_chunks, 0};
+    if (several) heavy[heavy_base + h] = HeavyRow{row, partial_base + p0, n_chunks, 0};
 }
 
 __global__ void mark_rows_kernel(const int32_t* __restrict__ rows, long long n, uint8_t* __restrict__ covered) {

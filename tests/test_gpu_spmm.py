@@ -7,6 +7,8 @@ import scipy.sparse as sp
 
 from oracle import liteform_oracle as O
 
+from liteform_ae_amd.format_matrix_market import MTX
+
 from helpers import skewed_matrix
 
 pytestmark = pytest.mark.gpu
@@ -104,6 +106,20 @@ def test_very_long_rows_are_split_into_chunks(fa, torch, feat, b_dtype):
     for widths in ([[1, 2, 4, 8, 16]], [[8, 1024]]):
         _, info = check(fa, torch, g, widths, feat, b_dtype)
         assert info["heavy_rows"] >= 2 and info["partial_rows"] >= 2 * 8
+
+
+def test_every_row_takes_the_cooperative_path(fa, torch):
+    """A matrix of long rows only: every lane of the table-building pass owns a heavy row,
+    single-chunk rows (<= 2048 slots) and multi-chunk rows mixed."""
+    rng = np.random.default_rng(91)
+    nr, nc = 700, 6000
+    deg = rng.integers(300, 5000, size=nr)
+    rows = np.repeat(np.arange(nr), deg)
+    cols = np.concatenate([rng.choice(nc, size=d, replace=False) for d in deg])
+    g = MTX.from_coo(rows, cols, (nr, nc), data=rng.uniform(-1, 1, size=len(rows)).astype(np.float32))
+    for widths in ([[16]], [[256, 1024]], [[8, 64], [1024]]):
+        _, info = check(fa, torch, g, widths, 64, seed=5)
+        assert info["heavy_rows"] > 0 and info["partial_rows"] > 0
 
 
 @pytest.mark.parametrize("feat,b_dtype", [(768, "f32"), (1024, "f32"), (1024, "bf16"), (32, "bf16"), (160, "f32")])
