@@ -48,6 +48,38 @@ def test_statistics_full_size(big):
         assert sum(int(hist[0, m]) for m in range(2048) if m >> k & 1) == len(cols_k)
 
 
+@pytest.mark.parametrize("parts", [1, 2])
+def test_column_set_histogram_full_size(big, parts):
+    """Every bin of the class-mask histogram against numpy: per partition and class, the
+    columns touched by rows of that class, then one mask per column."""
+    wl, fa, torch = big
+    g = wl.matrix
+    rows, cols = wl.shape
+    stats, hist = fa.bucket_statistics(g, parts)
+    indptr, indices, _ = g.adj_tensors("csr")
+    psize = -(-cols // parts)
+    row_of = np.repeat(np.arange(rows, dtype=np.int32), np.diff(indptr))
+    part_of = indices // psize
+    for p in range(parts):
+        sel = part_of == p
+        idx_p, row_p = indices[sel], row_of[sel]
+        deg = np.bincount(row_p, minlength=rows).astype(np.int64)
+        cls = np.where(deg <= 1, 0, np.ceil(np.log2(np.maximum(deg, 1))).astype(np.int64))
+        cls = np.minimum(cls, 10)
+        cls_of_nnz = cls[row_p]
+        mask = np.zeros(cols, dtype=np.int64)
+        for k in range(11):
+            touched = np.zeros(cols, dtype=bool)
+            touched[idx_p[cls_of_nnz == k]] = True
+            mask[touched] |= 1 << k
+        lo, hi = p * psize, min(cols, (p + 1) * psize)
+        want = np.bincount(mask[lo:hi], minlength=2048)
+        np.testing.assert_array_equal(hist[p], want)
+        for k in range(11):
+            m = (cls == k) & (deg > 0)
+            assert stats[p, k, 1] == deg[m].sum() and stats[p, k, 2] == m.sum()
+
+
 @pytest.mark.parametrize("parts,model", [(1, "reference"), (2, "gfx950")])
 def test_format_round_trip_full_size(big, parts, model):
     wl, fa, torch = big
