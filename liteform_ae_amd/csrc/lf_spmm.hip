@@ -411,9 +411,10 @@ __device__ __forceinline__ void ell_tile_segments_balanced(const Group& g, long 
             float v[kUnroll];
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
-                const int2 cv = rp[j + u];
-                c[u] = j + u < len ? cv.x : c0;
-                v[u] = __int_as_float(cv.y);
+                const bool in = j + u < len;          // W may be below kUnroll: stay inside the row
+                const int2 cv = rp[in ? j + u : 0];
+                c[u] = in ? cv.x : c0;
+                v[u] = in ? __int_as_float(cv.y) : 0.f;
             }
             gather_fma<kUnroll, LPR, CH, BT>(a.B, ln, c, v, acc);
         }
@@ -1133,6 +1134,15 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             const bool staged = fit >= sw;
             g.type = staged ? (is_multi[k] ? kEllSeg : kEll) : kSeg;
             g.rows_per_tile = staged ? std::min(kTileRows, fit) : std::max(sw, fit);
+            if (staged) {
+                // a small bucket is cut into more, shorter tiles so that it still spreads over
+                // the CUs: at least one pass of every sub-wave (8 rows at a time in the
+                // narrow-bucket code), aiming at four tiles per CU
+                const int unit = sw * (b.width < kUnroll ? kUnroll / b.width : 1);
+                const long long want = lf::ceil_div(b.num_ell_rows, (long long)4 * plan->num_cus);
+                const long long rows = std::max<long long>(unit, lf::ceil_div(want, (long long)unit) * unit);
+                g.rows_per_tile = (int)std::min<long long>(g.rows_per_tile, rows);
+            }
             if (g.type == kEllSeg) {
                 const long long part_bytes = (long long)g.rows_per_tile * feat_size * 4;
                 if (part_bytes <= kPartBytesMax) {

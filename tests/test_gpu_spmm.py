@@ -99,6 +99,16 @@ def test_folded_configurations_split_rows_over_ell_rows(fa, torch, feat, b_dtype
             assert info["lds_bytes"] > static_lds, (widths, info)
 
 
+@pytest.mark.parametrize("feat,b_dtype", [(32, "f32"), (64, "f32"), (128, "f32"), (256, "f32"), (128, "bf16")])
+def test_small_matrix_with_narrow_row_splitting_bucket(fa, torch, feat, b_dtype):
+    """Few rows, widest bucket of 1, 2 or 4 slots: short tiles, so the per-ELL-row sums of a
+    split row go through LDS with fewer slots per row than gathers in flight."""
+    rng = np.random.default_rng(700 + feat)
+    g = skewed_matrix(rng, 300, 400, mean_deg=5, heavy_rows=2, heavy_len=90)
+    for widths in ([[1]], [[2]], [[4]], [[1, 2]], [[2, 4]], [[1], [2]], [[4], [1, 2]]):
+        check(fa, torch, g, widths, feat, b_dtype, seed=feat)
+
+
 @pytest.mark.parametrize("feat,b_dtype", [(32, "f32"), (128, "f32"), (512, "bf16")])
 def test_very_long_rows_are_split_into_chunks(fa, torch, feat, b_dtype):
     rng = np.random.default_rng(77)
