@@ -1287,7 +1287,10 @@ int lf_spmm_time_ms(lf_spmm_plan* plan, const void* d_B, float* d_C, int32_t war
         if (int rc = lf_spmm_run(plan, d_B, d_C, stream)) return rc;
     hipEvent_t t0, t1;
     LF_HIP(hipEventCreate(&t0));
-    LF_HIP(hipEventCreate(&t1));
+    if (hipError_t e = hipEventCreate(&t1)) {
+        (void)hipEventDestroy(t0);
+        return lf::fail(LF_ERR_HIP, "hipEventCreate failed: %s", hipGetErrorString(e));
+    }
     int rc = LF_OK;
     for (int i = 0; i < repeat && rc == LF_OK; ++i) {
         if (d_flush && flush_bytes >= 4) {
