@@ -80,6 +80,14 @@ const char* lf_status_string(int status);
  * ------------------------------------------------------------------------------------ */
 size_t lf_stats_workspace_bytes(int64_t num_rows, int64_t num_cols, int32_t num_parts);
 
+/* Where lf_bucket_stats left the per-partition row bounds in its workspace:
+ * bounds[p][r] = first CSR position of row r whose column is >= p * ceil(num_cols / num_parts),
+ * p = 0..num_parts, int32 [num_parts + 1][num_rows].  NULL when num_parts == 1 (the row
+ * pointer is the bound).  Valid after lf_bucket_stats ran on that workspace with the same
+ * matrix and num_parts; lf_hyb_plan takes it as d_seg_bounds and then skips its own pass of
+ * binary searches over the column indices. */
+const int32_t* lf_stats_seg_bounds(const void* d_stats_workspace, int64_t num_rows, int32_t num_parts);
+
 int lf_bucket_stats(const int32_t* d_indptr, const int32_t* d_indices, const int32_t* d_seg_deg,
                     int64_t num_rows, int64_t num_cols, int32_t num_parts, int32_t width_limit,
                     void* d_workspace, size_t workspace_bytes,
@@ -142,6 +150,7 @@ int lf_search_bucket_config(const int64_t* h_stats, const int64_t* h_colhist, in
 size_t lf_hyb_workspace_bytes(int64_t num_rows, int32_t num_parts, int32_t total_buckets);
 
 int lf_hyb_plan(const int32_t* d_indptr, const int32_t* d_indices, const int32_t* d_seg_deg,
+                const int32_t* d_seg_bounds,
                 int64_t num_rows, int64_t num_cols, int32_t num_parts,
                 const int32_t* h_widths_flat, const int32_t* h_widths_off,
                 void* d_workspace, size_t workspace_bytes,

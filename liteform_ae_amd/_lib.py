@@ -57,7 +57,8 @@ SIGNATURES = {
                                           i32p, i32p, f64p, i32p]),
     "lf_hyb_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int32, C.c_int32]),
     "lf_hyb_layout": (C.c_int, [i64p, i32p, C.c_int32, i64p, i64p, i64p, i64p]),
-    "lf_hyb_plan": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int32, i32p, i32p, vp, C.c_size_t,
+    "lf_stats_seg_bounds": (vp, [vp, C.c_int64, C.c_int32]),
+    "lf_hyb_plan": (C.c_int, [vp, vp, vp, vp, C.c_int64, C.c_int64, C.c_int32, i32p, i32p, vp, C.c_size_t,
                               i64p, vp]),
     "lf_hyb_build": (C.c_int, [vp, vp, vp, vp, C.c_int64, C.c_int64, C.c_int32, i32p, i32p, i64p, vp,
                                C.c_size_t, vp, vp, vp, vp, vp, vp]),

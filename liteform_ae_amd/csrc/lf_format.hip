@@ -653,6 +653,11 @@ size_t lf_stats_workspace_bytes(int64_t num_rows, int64_t num_cols, int32_t num_
     return stats_layout(num_rows, num_cols, num_parts).total;
 }
 
+const int32_t* lf_stats_seg_bounds(const void* d_stats_workspace, int64_t num_rows, int32_t num_parts) {
+    if (d_stats_workspace == nullptr || num_parts <= 1 || num_rows <= 0) return nullptr;
+    return (const int32_t*)((const char*)d_stats_workspace + stats_layout(num_rows, 1, num_parts).bnd);
+}
+
 int lf_coo_degrees(const int32_t* d_coo_row, const int32_t* d_coo_col, int64_t nnz, int64_t num_rows,
                    int64_t num_cols, int32_t num_parts, int32_t* d_seg_deg, lf_stream_t stream) {
     hipStream_t s = (hipStream_t)stream;
@@ -753,7 +758,7 @@ int lf_hyb_layout(const int64_t* h_ell_rows, const int32_t* h_widths_flat, int32
 }
 
 int lf_hyb_plan(const int32_t* d_indptr, const int32_t* d_indices, const int32_t* d_seg_deg,
-                int64_t num_rows, int64_t num_cols, int32_t num_parts, const int32_t* h_widths_flat,
+                const int32_t* d_seg_bounds, int64_t num_rows, int64_t num_cols, int32_t num_parts, const int32_t* h_widths_flat,
                 const int32_t* h_widths_off, void* d_workspace, size_t workspace_bytes,
                 int64_t* h_ell_rows, lf_stream_t stream) {
     hipStream_t s = (hipStream_t)stream;
@@ -784,7 +789,10 @@ int lf_hyb_plan(const int32_t* d_indptr, const int32_t* d_indices, const int32_t
     LF_HIP(fill_u32(flags, 64, 0u, s));
     LF_HIP(fill_u32(totals, (int64_t)std::max(nb, 1) * 2, 0u, s));
     if (num_rows > 0) {
-        if (num_parts > 1) {
+        if (num_parts > 1 && d_seg_bounds) {       // bounds already known (the statistics pass made them)
+            LF_HIP(hipMemcpyAsync(bnd, d_seg_bounds, (size_t)(num_parts + 1) * num_rows * 4,
+                                  hipMemcpyDeviceToDevice, s));
+        } else if (num_parts > 1) {
             seg_bounds_kernel<<<L.nblk, kBlock, 0, s>>>(d_indptr, d_indices, num_rows, num_parts, psize, bnd);
             LF_HIP(hipGetLastError());
         }

@@ -105,6 +105,7 @@ class _DeviceCSR:
         self.all_ones = ones and self.nnz == self.coo_nnz
         self._g = g
         self._seg_deg = {}
+        self._stats_ws = {}          # num_parts -> statistics workspace holding the row bounds
 
     def seg_deg(self, num_parts: int):
         """Per-(partition,row) COO degrees on the device, or None when CSR lengths are the same."""
@@ -163,6 +164,10 @@ def bucket_statistics(g, num_parts: int, width_limit: int = WIDTH_LIMIT, with_co
                                    dev.num_rows, dev.num_cols, num_parts, width_limit,
                                    _lib.ptr(ws), nbytes, _lib.np_ptr(stats, C.c_int64),
                                    _lib.np_ptr(hist, C.c_int64) if with_columns else None, _stream()))
+    if num_parts > 1:
+        # the pass left the per-partition row bounds in its workspace; the slab builder takes
+        # them over instead of searching the column indices again
+        dev._stats_ws[num_parts] = ws
     return stats, hist
 
 
@@ -292,7 +297,9 @@ def build_hyb_format_device(g, bucket_widths, with_values: bool = True, with_mas
     ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device="cuda")
     stream = _stream()
     t0 = time.perf_counter()
-    _lib.check(lib.lf_hyb_plan(_lib.ptr(dev.indptr), _lib.ptr(dev.indices), _lib.ptr(seg_deg),
+    stats_ws = dev._stats_ws.get(P)
+    bounds = lib.lf_stats_seg_bounds(_lib.ptr(stats_ws), dev.num_rows, P) if stats_ws is not None else None
+    _lib.check(lib.lf_hyb_plan(_lib.ptr(dev.indptr), _lib.ptr(dev.indices), _lib.ptr(seg_deg), bounds,
                                dev.num_rows, dev.num_cols, P, _lib.np_ptr(flat, C.c_int32),
                                _lib.np_ptr(off, C.c_int32), _lib.ptr(ws), nbytes,
                                _lib.np_ptr(ell_rows, C.c_int64), stream))

@@ -53,8 +53,16 @@ def test_raw_abi_end_to_end(env):
     hb = lib.lf_hyb_workspace_bytes(rows, P, nb)
     hws = torch.empty(hb, dtype=torch.uint8, device="cuda")
     ell = np.zeros(nb, np.int64)
-    args = (d_ptr.data_ptr(), d_idx.data_ptr(), None, rows, cols, P, L.np_ptr(flat, C.c_int32), L.np_ptr(off, C.c_int32))
-    assert lib.lf_hyb_plan(*args, hws.data_ptr(), hb, L.np_ptr(ell, C.c_int64), None) == 0
+    # the statistics pass left the per-partition row bounds in its workspace; the plan takes them
+    bounds = lib.lf_stats_seg_bounds(ws.data_ptr(), rows, P)
+    assert (bounds is not None) == (P > 1)
+    ell_own = np.zeros(nb, np.int64)
+    args = (rows, cols, P, L.np_ptr(flat, C.c_int32), L.np_ptr(off, C.c_int32))
+    assert lib.lf_hyb_plan(d_ptr.data_ptr(), d_idx.data_ptr(), None, None, *args, hws.data_ptr(), hb,
+                           L.np_ptr(ell_own, C.c_int64), None) == 0
+    assert lib.lf_hyb_plan(d_ptr.data_ptr(), d_idx.data_ptr(), None, bounds, *args, hws.data_ptr(), hb,
+                           L.np_ptr(ell, C.c_int64), None) == 0
+    np.testing.assert_array_equal(ell, ell_own)     # same counts with its own pass over the indices
     ro, so = np.zeros(nb, np.int64), np.zeros(nb, np.int64)
     tr, ts = C.c_int64(), C.c_int64()
     assert lib.lf_hyb_layout(L.np_ptr(ell, C.c_int64), L.np_ptr(flat, C.c_int32), nb, L.np_ptr(ro, C.c_int64),
@@ -155,13 +163,13 @@ def test_error_paths_report_and_do_not_crash(env):
     flat = np.array([3], np.int32)
     off = np.array([0, 1], np.int32)
     ell = np.zeros(1, np.int64)
-    assert lib.lf_hyb_plan(indptr.data_ptr(), indices.data_ptr(), None, rows, cols, 1, L.np_ptr(flat, C.c_int32),
+    assert lib.lf_hyb_plan(indptr.data_ptr(), indices.data_ptr(), None, None, rows, cols, 1, L.np_ptr(flat, C.c_int32),
                            L.np_ptr(off, C.c_int32), ws.data_ptr(), 1 << 20, L.np_ptr(ell, C.c_int64),
                            None) == L.LF_ERR_INVALID
     flat = np.array([4, 2], np.int32)
     off = np.array([0, 2], np.int32)
     ell = np.zeros(2, np.int64)
-    assert lib.lf_hyb_plan(indptr.data_ptr(), indices.data_ptr(), None, rows, cols, 1, L.np_ptr(flat, C.c_int32),
+    assert lib.lf_hyb_plan(indptr.data_ptr(), indices.data_ptr(), None, None, rows, cols, 1, L.np_ptr(flat, C.c_int32),
                            L.np_ptr(off, C.c_int32), ws.data_ptr(), 1 << 20, L.np_ptr(ell, C.c_int64),
                            None) == L.LF_ERR_INVALID
     # SpMM: unsupported feature size, bad dtype, null output handle
