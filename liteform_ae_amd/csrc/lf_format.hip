@@ -352,7 +352,7 @@ hyb_scan_kernel(int32_t* __restrict__ blockcnt, int nblk, long long* __restrict_
     if (threadIdx.x == 0) totals[blockIdx.x] = s_carry;
 }
 
-// Fills the slabs.  One workgroup per 256 source rows, all column partitions in turn.
+// Fills the slabs.  One workgroup per 256 source rows, four column partitions at a time.
 //   * one thread per (row, partition) segment finds the segment's bucket and its first ELL
 //     row (per-wavefront counts per bucket - bit counts, or a shuffle scan where segments
 //     split - combined through LDS with a single barrier) and writes the rows / meta entries;
@@ -370,6 +370,7 @@ struct BucketOffsets {
 };
 
 constexpr int kFillUnroll = 4;
+constexpr int kPartGroup = 4;        // column partitions whose segments are walked together
 // four consecutive 32-bit values at a 4-byte aligned address (one 16-byte load)
 struct __attribute__((packed, aligned(4))) Packed4i { int x, y, z, w; };
 struct __attribute__((packed, aligned(4))) Packed4f { float x, y, z, w; };
@@ -380,108 +381,134 @@ hyb_fill_kernel(SegView v, const int32_t* __restrict__ seg_deg, const int32_t* _
                 const int32_t* __restrict__ indices, const float* __restrict__ values,
                 int32_t* __restrict__ out_rows, int32_t* __restrict__ out_meta,
                 int32_t* __restrict__ out_cols, float* __restrict__ out_vals, float* __restrict__ out_mask) {
+    // segment tables of the walk, entry t * pg + pp for row t and the pp-th partition of the
+    // group of pg <= kPartGroup partitions in hand: row-major, so the walk reads each row's CSR
+    // entries once and in order however many partitions cut it
+    constexpr int kSegs = kBlock * kPartGroup;
     __shared__ int s_cnt[kBlock / 64][LF_MAX_CLASSES + 1];
     // exclusive prefix of the padded segment lengths; 32 bits are enough: a segment is padded
     // by less than 1024 slots and the matrix holds fewer than 2^31 entries
-    __shared__ uint32_t s_off[kBlock + 1];
-    __shared__ long long s_dst[kBlock];        // first slab slot of each segment
+    __shared__ uint32_t s_off[kSegs + 1];
+    __shared__ long long s_dst[kSegs];         // first slab slot of each segment
+    __shared__ int s_start[kSegs];
+    __shared__ int s_fill[kSegs];
+    __shared__ uint32_t s_len[kSegs];
     __shared__ uint32_t s_wave[kBlock / 64];
-    __shared__ int s_start[kBlock];
-    __shared__ int s_fill[kBlock];
-    __shared__ uint32_t s_len[kBlock];
     const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
-    for (int p = 0; p < v.parts; ++p) {
-        const int32_t* w = wtab + p * kWtabStride;
-        const int n = w[0];
-        const int kbase = w[12];
-        int start = 0, fill = 0, mine = -1, width = 1, n_ell = 0;
-        if (r < v.rows && n > 0) {
-            seg_range(v, r, p, start, fill);
-            if (fill > 0) {
-                const int deg = seg_deg ? seg_deg[(int64_t)p * v.rows + r] : fill;
-                mine = pick_bucket(w, n, deg);
-                width = w[1 + mine];
-                n_ell = (fill + width - 1) / width;
-            }
-        }
-        // ELL rows of the same bucket that precede this segment inside its wavefront.  Only the
-        // widest bucket splits segments; where every segment is one ELL row a bit count does it.
-        int in_wave = 0;
-        for (int b = 0; b < n; ++b) {
-            const unsigned long long members = __ballot(mine == b);
-            if (__ballot(mine == b && n_ell != 1) == 0) {
-                if (mine == b) in_wave = __popcll(members & ((1ull << lane) - 1ull));
-                if (lane == 0) s_cnt[wave][b] = __popcll(members);
-            } else {
-                const int x = mine == b ? n_ell : 0;
-                int incl = x;
-                for (int d = 1; d < 64; d <<= 1) {
-                    const int y = __shfl_up(incl, d);
-                    if (lane >= d) incl += y;
+    for (int p0 = 0; p0 < v.parts; p0 += kPartGroup) {
+        const int pg = min(kPartGroup, v.parts - p0);
+        uint32_t vl[kPartGroup];
+#pragma unroll
+        for (int pp = 0; pp < kPartGroup; ++pp) {
+            vl[pp] = 0;
+            if (pp >= pg) continue;                    // uniform
+            const int p = p0 + pp;
+            const int32_t* w = wtab + p * kWtabStride;
+            const int n = w[0];
+            const int kbase = w[12];
+            int start = 0, fill = 0, mine = -1, width = 1, n_ell = 0;
+            if (r < v.rows && n > 0) {
+                seg_range(v, r, p, start, fill);
+                if (fill > 0) {
+                    const int deg = seg_deg ? seg_deg[(int64_t)p * v.rows + r] : fill;
+                    mine = pick_bucket(w, n, deg);
+                    width = w[1 + mine];
+                    n_ell = (fill + width - 1) / width;
                 }
-                if (mine == b) in_wave = incl - x;
-                if (lane == 63) s_cnt[wave][b] = incl;
             }
+            // ELL rows of the same bucket that precede this segment inside its wavefront.  Only
+            // the widest bucket splits segments; where every segment is one ELL row a bit count
+            // does it.
+            int in_wave = 0;
+            for (int b = 0; b < n; ++b) {
+                const unsigned long long members = __ballot(mine == b);
+                if (__ballot(mine == b && n_ell != 1) == 0) {
+                    if (mine == b) in_wave = __popcll(members & ((1ull << lane) - 1ull));
+                    if (lane == 0) s_cnt[wave][b] = __popcll(members);
+                } else {
+                    const int x = mine == b ? n_ell : 0;
+                    int incl = x;
+                    for (int d = 1; d < 64; d <<= 1) {
+                        const int y = __shfl_up(incl, d);
+                        if (lane >= d) incl += y;
+                    }
+                    if (mine == b) in_wave = incl - x;
+                    if (lane == 63) s_cnt[wave][b] = incl;
+                }
+            }
+            __syncthreads();
+            long long first = 0;      // flat ELL-row index of this segment's first ELL row
+            long long dst = 0;
+            if (mine >= 0) {
+                int wave_off = 0;
+                for (int wv = 0; wv < wave; ++wv) wave_off += s_cnt[wv][mine];
+                const BucketOffsets bo = offs[kbase + mine];
+                const long long local = (long long)blockoff[(int64_t)(kbase + mine) * nblk + blockIdx.x] + wave_off + in_wave;
+                first = bo.row_off + local;
+                dst = bo.slot_off + local * width;
+            }
+            const uint32_t slen = (uint32_t)n_ell * (uint32_t)width;   // slots of the segment's ELL rows
+            vl[pp] = (slen + 3u) & ~3u;
+            const int idx = threadIdx.x * pg + pp;
+            s_dst[idx] = dst;
+            s_start[idx] = start;
+            s_fill[idx] = fill;
+            s_len[idx] = slen;
+
+            const bool is_long = n_ell > 8;
+            if (n_ell > 0 && !is_long) {
+                for (int i = 0; i < n_ell; ++i) {
+                    const int len = min(width, fill - i * width);
+                    out_rows[first + i] = (int32_t)r;
+                    out_meta[first + i] = make_meta(len, i, n_ell);
+                }
+            }
+            unsigned long long pending = __ballot(is_long);
+            while (pending) {
+                const int src = __ffsll((long long)pending) - 1;
+                pending &= pending - 1;
+                const long long f0 = __shfl(first, src);
+                const int fl = __shfl(fill, src);
+                const int wd = __shfl(width, src);
+                const int ne = __shfl(n_ell, src);
+                const int rr = (int)((int64_t)blockIdx.x * kBlock + (wave << 6) + src);
+                for (int i = lane; i < ne; i += 64) {
+                    const int len = min(wd, fl - i * wd);
+                    out_rows[f0 + i] = rr;
+                    out_meta[f0 + i] = make_meta(len, i, ne);
+                }
+            }
+            __syncthreads();          // s_cnt is rewritten for the next partition
         }
-        // padded length of the segment and its prefix inside the wavefront
-        const uint32_t slen = (uint32_t)n_ell * (uint32_t)width;   // slots of the segment's ELL rows
-        const uint32_t vlen = (slen + 3u) & ~3u;
-        uint32_t vincl = vlen;
+
+        // exclusive prefix of the padded lengths over (row, partition)
+        uint32_t mine_total = 0;
+#pragma unroll
+        for (int pp = 0; pp < kPartGroup; ++pp) mine_total += vl[pp];
+        uint32_t vincl = mine_total;
         for (int d = 1; d < 64; d <<= 1) {
             const uint32_t y = __shfl_up(vincl, d);
             if (lane >= d) vincl += y;
         }
         if (lane == 63) s_wave[wave] = vincl;
         __syncthreads();
-        long long first = 0;      // flat ELL-row index of this segment's first ELL row
-        long long dst = 0;
-        if (mine >= 0) {
-            int wave_off = 0;
-            for (int wv = 0; wv < wave; ++wv) wave_off += s_cnt[wv][mine];
-            const BucketOffsets bo = offs[kbase + mine];
-            const long long local = (long long)blockoff[(int64_t)(kbase + mine) * nblk + blockIdx.x] + wave_off + in_wave;
-            first = bo.row_off + local;
-            dst = bo.slot_off + local * width;
-        }
-        uint32_t voff = vincl - vlen;
+        uint32_t voff = vincl - mine_total;
         for (int wv = 0; wv < wave; ++wv) voff += s_wave[wv];
-        s_off[threadIdx.x] = voff;
-        s_dst[threadIdx.x] = dst;
-        s_start[threadIdx.x] = start;
-        s_fill[threadIdx.x] = fill;
-        s_len[threadIdx.x] = slen;
-        if (threadIdx.x == kBlock - 1) s_off[kBlock] = voff + vlen;
-
-        const bool is_long = n_ell > 8;
-        if (n_ell > 0 && !is_long) {
-            for (int i = 0; i < n_ell; ++i) {
-                const int len = min(width, fill - i * width);
-                out_rows[first + i] = (int32_t)r;
-                out_meta[first + i] = make_meta(len, i, n_ell);
-            }
+#pragma unroll
+        for (int pp = 0; pp < kPartGroup; ++pp) {
+            if (pp < pg) s_off[threadIdx.x * pg + pp] = voff;
+            voff += vl[pp];
         }
-        unsigned long long pending = __ballot(is_long);
-        while (pending) {
-            const int src = __ffsll((long long)pending) - 1;
-            pending &= pending - 1;
-            const long long f0 = __shfl(first, src);
-            const int fl = __shfl(fill, src);
-            const int wd = __shfl(width, src);
-            const int ne = __shfl(n_ell, src);
-            const int rr = (int)((int64_t)blockIdx.x * kBlock + (wave << 6) + src);
-            for (int i = lane; i < ne; i += 64) {
-                const int len = min(wd, fl - i * wd);
-                out_rows[f0 + i] = rr;
-                out_meta[f0 + i] = make_meta(len, i, ne);
-            }
-        }
+        if (threadIdx.x == kBlock - 1) s_off[kBlock * pg] = voff;
         __syncthreads();
 
         // groups of four consecutive slots; the prefix sums are multiples of four, so a group
         // never straddles two segments
-        const uint32_t total = s_off[kBlock];
+        const int n_seg = kBlock * pg;
+        const int steps = 8 + (pg > 1) + (pg > 2);       // ceil(log2(n_seg))
+        const uint32_t total = s_off[n_seg];
         for (uint32_t j0 = 0; j0 < total; j0 += kBlock * kFillUnroll * 4) {
             long long at[kFillUnroll];
             int len[kFillUnroll];                     // slots of the group inside its segment (0: none)
@@ -496,9 +523,8 @@ hyb_fill_kernel(SegView v, const int32_t* __restrict__ seg_deg, const int32_t* _
                 x[u] = make_float4(0.f, 0.f, 0.f, 0.f);
                 m[u] = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (j < total) {
-                    int lo = 0, hi = kBlock - 1;       // last segment whose offset is <= j
-#pragma unroll
-                    for (int step = 0; step < 8; ++step) {
+                    int lo = 0, hi = n_seg - 1;        // last segment whose offset is <= j
+                    for (int step = 0; step < steps; ++step) {
                         const int mid = (lo + hi + 1) >> 1;
                         if (s_off[mid] <= j) lo = mid; else hi = mid - 1;
                     }
@@ -545,7 +571,7 @@ hyb_fill_kernel(SegView v, const int32_t* __restrict__ seg_deg, const int32_t* _
                 }
             }
         }
-        __syncthreads();          // the tables are rewritten for the next partition
+        __syncthreads();          // the tables are rewritten for the next group of partitions
     }
 }
 
