@@ -82,8 +82,8 @@ def test_every_width_path(fa, torch, widths):
     check(fa, torch, g, widths, 128)
 
 
-@pytest.mark.parametrize("feat,b_dtype", [(32, "f32"), (64, "f32"), (128, "f32"), (256, "f32"), (64, "bf16"),
-                                          (256, "bf16")])
+@pytest.mark.parametrize("feat,b_dtype", [(32, "f32"), (64, "f32"), (128, "f32"), (256, "f32"), (512, "f32"),
+                                          (64, "bf16"), (256, "bf16"), (1024, "bf16")])
 def test_folded_configurations_split_rows_over_ell_rows(fa, torch, feat, b_dtype):
     """Widest bucket narrower than most rows: segments of 2..8 ELL rows (many cross a tile
     boundary), summed row by row through LDS where the tile's partial sums fit."""
@@ -94,7 +94,8 @@ def test_folded_configurations_split_rows_over_ell_rows(fa, torch, feat, b_dtype
     plain.close()
     for widths in ([[8]], [[16]], [[32]], [[1, 2, 4, 8, 16, 32]], [[64]], [[4, 16], [2, 32]]):
         _, info = check(fa, torch, g, widths, feat, b_dtype, seed=feat)
-        rows_per_tile = max(512, 64 * 256 // (feat // (8 if b_dtype == "bf16" else 4))) // widths[0][-1]
+        lpr = min(64, feat // (8 if b_dtype == "bf16" else 4))
+        rows_per_tile = max(512, 64 * 256 // lpr) // widths[0][-1]
         if rows_per_tile * feat * 4 <= 16384 and len(widths) == 1:
             assert info["lds_bytes"] > static_lds, (widths, info)
 
