@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused hyb SpMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3] [--feat 128] [--parts 1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3] [--feat 128] [--parts 1] [--windows 1]
 
 A step is one SpMM  C = A_hyb . B  over the whole synthetic matrix, with A's hyb slabs, B and
 C resident in HBM.  The default workload is the 2.45M-row power-law graph at N = 128, the
@@ -10,8 +10,8 @@ configuration the headline metric is quoted on.  Prints one JSON line:
   value            GFLOP/s = 2 * nnz * N / t, from the wall time of K back-to-back steps
   roofline         HBM: algorithmic bytes per step / average kernel time of a step measured
                    with HIP events on the launch stream (a step is one launch per column
-                   partition; bytes and time are both summed over them, so the ratio is also
-                   the per-launch one); traffic = L2<->fabric bytes per step from rocprofv3
+                   partition and feature window; bytes and time are both summed over them, so
+                   the ratio is also the per-launch one); traffic = L2<->fabric bytes per step from rocprofv3
                    counters when a measurement is on file
   format_compose   bucket-width search and slab build times (GPU), reported beside it
   cpu_baseline     scipy CSR @ dense (the reference's own CPU product, one thread) on a
@@ -54,8 +54,8 @@ MEASURED_TRAFFIC = {
 }
 
 
-def recorded_traffic(workload, feat, parts):
-    return MEASURED_TRAFFIC.get(f"{workload}/N{feat}/P{parts}")
+def recorded_traffic(workload, feat, parts, windows):
+    return MEASURED_TRAFFIC.get(f"{workload}/N{feat}/P{parts}" + (f"/W{windows}" if windows > 1 else ""))
 
 
 def cpu_baseline(wl, B_host, feat, budget_s=20.0):
@@ -178,6 +178,8 @@ def main():
     ap.add_argument("--feat", type=int, default=0, help="dense columns N (default: the workload's)")
     ap.add_argument("--parts", type=int, default=0,
                     help="column partitions (default: the workload's; measured choice where it names none)")
+    ap.add_argument("--windows", type=int, default=0,
+                    help="feature windows per step (0 = by measurement together with the partitions)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the matrix (testing only)")
     ap.add_argument("--cost-model", default="gfx950", choices=["reference", "gfx950"],
                     help="cost function of the bucket-width search (the reference's, or the MI355X one)")
@@ -232,12 +234,15 @@ def main():
     torch.cuda.synchronize()
     ingest_ms = (time.perf_counter() - t0) * 1e3
     part_timings = None
-    if not parts:                           # the workload leaves the partition count open
+    windows = args.windows
+    if not parts or not windows:            # left open: partition count and feature windows by measurement
         t0 = time.perf_counter()
-        parts, part_timings = fa.choose_num_partitions(g, feat, wl.b_dtype, cost_model=args.cost_model,
-                                                       return_timings=True)
-        print(f"[bench] partition count chosen by measurement: {parts} from {part_timings} "
-              f"({time.perf_counter() - t0:.2f} s)", file=sys.stderr, flush=True)
+        (parts, windows), shape_timings = fa.choose_launch_shape(
+            g, feat, wl.b_dtype, candidates=(parts,) if parts else (1, 2, 3, 4),
+            windows=(windows,) if windows else None, cost_model=args.cost_model, return_timings=True)
+        part_timings = {f"P{p}xW{w}": round(t, 4) for (p, w), t in shape_timings.items()}
+        print(f"[bench] launch shape chosen by measurement: {parts} partition(s) x {windows} feature window(s) "
+              f"from {part_timings} ({time.perf_counter() - t0:.2f} s)", file=sys.stderr, flush=True)
     cfg_obj = fa.CostModelSettings(feat, parts, cost_model=args.cost_model)
     fa.search_bucket_config(g, parts, cfg_obj)            # warm
     t0 = time.perf_counter()
@@ -251,10 +256,10 @@ def main():
     t0 = time.perf_counter()
     fmt = fa.build_hyb_format_device(g, config)
     build_ms = (time.perf_counter() - t0) * 1e3
-    fa.HybSpMM(fmt, feat, wl.b_dtype).close()             # warm
+    fa.HybSpMM(fmt, feat, wl.b_dtype, windows=windows).close()     # warm
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    plan = fa.HybSpMM(fmt, feat, wl.b_dtype)
+    plan = fa.HybSpMM(fmt, feat, wl.b_dtype, windows=windows)
     torch.cuda.synchronize()
     plan_ms = (time.perf_counter() - t0) * 1e3
     print(f"[bench] config {config}; search {search_ms:.2f} ms, build {build_ms:.2f} ms, "
@@ -291,7 +296,7 @@ def main():
     algo = algorithmic_bytes(nnz, rows, cols, feat, b_bytes)
     gath = gather_bytes(nnz, rows, feat, b_bytes)
     achieved = algo / (kernel_ms * 1e-3) / 1e9
-    traffic = recorded_traffic(wl.name if args.scale == 1.0 else "", feat, parts)
+    traffic = recorded_traffic(wl.name if args.scale == 1.0 else "", feat, parts, windows)
 
     result = {
         "metric": "SpMM GFLOP/s & % HBM roofline at N=128; format-compose ms",
@@ -308,9 +313,9 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": f"{wl.name}: {wl.description}" + ("" if args.scale == 1.0 else f" (scale {args.scale})"),
-            "rows": rows, "cols": cols, "nnz": nnz, "feat_size": feat, "num_parts": parts,
+            "rows": rows, "cols": cols, "nnz": nnz, "feat_size": feat, "num_parts": parts, "feature_windows": windows,
             "bucket_widths": config, "cost_model": args.cost_model,
-            "num_parts_candidates_ms": part_timings,
+            "launch_shape_candidates_ms": part_timings,
         },
         "roofline": {
             "bound": "hbm",
@@ -319,7 +324,7 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 5),
             "traffic": traffic,
-            "launches_per_step": parts,
+            "launches_per_step": parts * windows,
             "kernel_ms": round(kernel_ms, 4),
             "kernel_ms_min": round(float(np.min(ev_ms)), 4),
             "kernel_ms_cold": round(float(np.mean(ev_cold_ms)), 4),

@@ -197,6 +197,20 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
 int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t stream);
 int lf_spmm_destroy(lf_spmm_plan* plan);
 
+/* Feature windows.  A plan created for feat_size features can cover operands n_windows times
+ * as wide: B [num_cols][n_windows * feat_size], C [num_rows][n_windows * feat_size]; a run then
+ * makes one pass per window of feat_size features (all partitions inside), reading and
+ * writing only that window's columns.  Features are independent, so the result is that of a
+ * plan created for the full width, except that rows split over several ELL rows or reduced
+ * cooperatively are summed in pieces whose size follows the lane count (same tolerance, not
+ * the same bits).  Narrow
+ * windows pay off when B is much larger than the memory-side cache: the part of B that one
+ * pass touches is a fraction of the whole, and C is still written once (cfg3, 2.45M rows,
+ * N = 128: 6.27 ms in two windows of 64 against 6.94 ms in one pass).  Applies to lf_spmm_run and lf_spmm_time_ms; the default is one window.  No
+ * counterpart in the reference (its feature tiling lives inside one launch,
+ * format_algos.py:491-520). */
+int lf_spmm_set_windows(lf_spmm_plan* plan, int32_t n_windows);
+
 /* h_info[0..7] = tiles, workgroups per launch, launches per run, LDS bytes per workgroup,
  * heavy (split) segments, partial rows, rows cleared by partition 0, reserved. */
 int lf_spmm_info(const lf_spmm_plan* plan, int64_t* h_info);

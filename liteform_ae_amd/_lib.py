@@ -66,6 +66,7 @@ SIGNATURES = {
                                  C.c_int64, C.c_int32, C.c_int32, vp]),
     "lf_spmm_run": (C.c_int, [vp, vp, vp, vp]),
     "lf_spmm_destroy": (C.c_int, [vp]),
+    "lf_spmm_set_windows": (C.c_int, [vp, C.c_int32]),
     "lf_spmm_info": (C.c_int, [vp, i64p]),
     "lf_spmm_time_ms": (C.c_int, [vp, vp, vp, C.c_int32, C.c_int32, vp, C.c_size_t, f32p, vp]),
     "lf_csr_spmm": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int32, C.c_int32, vp, vp, vp]),

@@ -102,7 +102,8 @@ struct LaunchArgs {
     const Group* groups;
     int n_groups;
     int accumulate;               // 0: C = result, 1: C += result
-    int feat;                     // N
+    int feat;                     // N: features computed by the launch
+    int ldb, ldc;                 // row strides of B and C in elements (N, or more for a feature window)
     int pad_;
     const void* B;
     float* C;
@@ -148,10 +149,12 @@ template <int CH, int VEC> struct Acc {
 // Position of a lane inside the feature dimension.
 template <int LPR, int CH, int VEC> struct Lane {
     int sl;                 // lane inside the sub-wave
-    int feat;               // N
+    int feat;               // N: features this launch computes
+    int ldb, ldc;           // elements between consecutive rows of B and of C (>= N)
     int f[CH];              // first feature of each chunk (clamped to 0 when outside N)
     bool on[CH];
-    __device__ __forceinline__ Lane(int sl_, int feat_) : sl(sl_), feat(feat_) {
+    __device__ __forceinline__ Lane(int sl_, int feat_, int ldb_, int ldc_)
+        : sl(sl_), feat(feat_), ldb(ldb_), ldc(ldc_) {
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int f0 = (c * LPR + sl_) * VEC;
@@ -171,7 +174,7 @@ __device__ __forceinline__ void gather_fma(const void* B, const Lane<LPR, CH, De
     for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int c = 0; c < CH; ++c)
-            Dense<BT>::load(B, (size_t)(uint32_t)col[u] * (size_t)ln.feat + ln.f[c], x[u][c]);
+            Dense<BT>::load(B, (size_t)(uint32_t)col[u] * (size_t)ln.ldb + ln.f[c], x[u][c]);
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -186,7 +189,7 @@ __device__ __forceinline__ void store_row(float* C, int row, const Lane<LPR, CH,
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         if (!ln.on[c]) continue;
-        float* dst = C + (size_t)row * ln.feat + ln.f[c];
+        float* dst = C + (size_t)row * ln.ldc + ln.f[c];
 #pragma unroll
         for (int i = 0; i < VEC; i += 4) {
             float4 o = make_float4(acc.v[c][i], acc.v[c][i + 1], acc.v[c][i + 2], acc.v[c][i + 3]);
@@ -242,7 +245,7 @@ __device__ __forceinline__ void ell_tile_narrow(const int2* s_pairs, const int2*
     constexpr int VEC = Dense<BT>::kVec;
     constexpr int SW = kWG / LPR;
     constexpr int RPI = kUnroll / W;
-    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const Lane<LPR, CH, VEC> ln(sl, a.feat, a.ldb, a.ldc);
     for (int r0 = sw * RPI; r0 < n; r0 += SW * RPI) {
         Acc<CH, VEC> acc[RPI];
         int c[kUnroll];
@@ -266,7 +269,7 @@ __device__ __forceinline__ void ell_tile_narrow(const int2* s_pairs, const int2*
             for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
                 for (int cc = 0; cc < CH; ++cc)
-                    Dense<BT>::load(a.B, (size_t)(uint32_t)c[u] * (size_t)ln.feat + ln.f[cc], x[u][cc]);
+                    Dense<BT>::load(a.B, (size_t)(uint32_t)c[u] * (size_t)ln.ldb + ln.f[cc], x[u][cc]);
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
@@ -304,7 +307,7 @@ __device__ __forceinline__ void ell_tile_wide(const int2* s_pairs, const int2* s
                                               const LaunchArgs& a, int sw, int sl) {
     constexpr int VEC = Dense<BT>::kVec;
     constexpr int SW = kWG / LPR;
-    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const Lane<LPR, CH, VEC> ln(sl, a.feat, a.ldb, a.ldc);
     for (int r = sw; r < n; r += SW) {
         const int2 rm = s_rm[r];
         const int len = rm.y & kMetaLenMask;
@@ -337,7 +340,7 @@ __device__ __forceinline__ void ell_tile_segments(const Group& g, long long e0, 
                                                   const int2* s_rm, int n, const LaunchArgs& a, int* s_next,
                                                   int sl) {
     constexpr int VEC = Dense<BT>::kVec;
-    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const Lane<LPR, CH, VEC> ln(sl, a.feat, a.ldb, a.ldc);
     const int log_w = g.log_w;
     // Segments differ in length and continuation rows carry no work, so the sub-waves take
     // the tile's ELL rows from a shared counter as they become free instead of by a fixed
@@ -392,7 +395,7 @@ __device__ __forceinline__ void ell_tile_segments_balanced(const Group& g, long 
                                                            float* s_part, int sw, int sl) {
     constexpr int VEC = Dense<BT>::kVec;
     constexpr int SW = kWG / LPR;
-    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const Lane<LPR, CH, VEC> ln(sl, a.feat, a.ldb, a.ldc);
     const int log_w = g.log_w;
     for (int r = sw; r < n; r += SW) {
         const int2 rm = s_rm[r];
@@ -513,7 +516,7 @@ __device__ __forceinline__ void run_seg_tile(const Group& g, long long tile, con
     constexpr int SW = kWG / LPR;
     const int tid = threadIdx.x;
     const int sw = tid / LPR, sl = tid % LPR;
-    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const Lane<LPR, CH, VEC> ln(sl, a.feat, a.ldb, a.ldc);
     const long long e0 = tile * g.rows_per_tile;
     const int n = (int)min((long long)g.rows_per_tile, g.n_items - e0);
     for (int r = sw; r < n; r += SW) {
@@ -537,7 +540,7 @@ __device__ __forceinline__ void run_zero_tile(const Group& g, long long tile, co
     constexpr int SW = kWG / LPR;
     const int tid = threadIdx.x;
     const int sw = tid / LPR, sl = tid % LPR;
-    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const Lane<LPR, CH, VEC> ln(sl, a.feat, a.ldb, a.ldc);
     const long long e0 = tile * g.rows_per_tile;
     const int n = (int)min((long long)g.rows_per_tile, g.n_items - e0);
     Acc<CH, VEC> zero;
@@ -554,7 +557,7 @@ __device__ __forceinline__ void run_chunk_tile(const Group& g, long long tile, f
     constexpr int SW = kWG / LPR;
     const int tid = threadIdx.x;
     const int sw = tid / LPR, sl = tid % LPR;
-    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const Lane<LPR, CH, VEC> ln(sl, a.feat, a.ldb, a.ldc);
     const Chunk ck = g.chunks[tile];
     int per = (ck.n_slots + SW - 1) / SW;
     per = (per + LPR - 1) / LPR * LPR;
@@ -642,7 +645,7 @@ spmm_finalize_kernel(const HeavyRow* __restrict__ heavy, int n_heavy, LaunchArgs
     constexpr int VEC = Dense<BT>::kVec;
     constexpr int SW = kWG / LPR;
     const int sw = threadIdx.x / LPR, sl = threadIdx.x % LPR;
-    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const Lane<LPR, CH, VEC> ln(sl, a.feat, a.ldb, a.ldc);
     for (int h = blockIdx.x * SW + sw; h < n_heavy; h += gridDim.x * SW) {
         const HeavyRow hr = heavy[h];
         Acc<CH, VEC> acc;
@@ -668,7 +671,7 @@ csr_spmm_kernel(const int32_t* __restrict__ indptr, const int32_t* __restrict__ 
     constexpr int VEC = Dense<BT>::kVec;
     constexpr int SW = kWG / LPR;
     const int sw = threadIdx.x / LPR, sl = threadIdx.x % LPR;
-    const Lane<LPR, CH, VEC> ln(sl, a.feat);
+    const Lane<LPR, CH, VEC> ln(sl, a.feat, a.ldb, a.ldc);
     for (long long r = (long long)blockIdx.x * SW + sw; r < n_rows; r += (long long)gridDim.x * SW) {
         const int lo = indptr[r], hi = indptr[r + 1];
         Acc<CH, VEC> acc;
@@ -832,6 +835,7 @@ struct lf_spmm_plan {
     int feat = 0, b_dtype = 0, num_parts = 0;
     int64_t num_rows = 0, num_cols = 0;
     int lpr = 0, ch = 0;
+    int windows = 1;                 // feature windows of `feat` features each that a run covers
     int device = 0, num_cus = 0, grid = 0;
     struct Launch {
         int group_begin = 0, n_groups = 0, grid = 0;
@@ -1231,26 +1235,40 @@ int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t str
     LF_REQUIRE((uintptr_t)d_B % 16 == 0 && (uintptr_t)d_C % 16 == 0, LF_ERR_INVALID, "B and C must be 16-byte aligned");
     KernelSet ks;
     if (int rc = select_kernels(plan->lpr, plan->ch, plan->b_dtype, &ks)) return rc;
-    for (int p = 0; p < plan->num_parts; ++p) {
-        const lf_spmm_plan::Launch& L = plan->launches[p];
-        if (L.n_groups == 0) continue;
-        LaunchArgs a{};
-        a.groups = plan->d_groups + L.group_begin;
-        a.n_groups = L.n_groups;
-        a.accumulate = p > 0 ? 1 : 0;
-        a.feat = plan->feat;
-        a.B = d_B;
-        a.C = d_C;
-        a.partials = plan->d_partials;
-        ks.tiles<<<L.grid, kWG, L.dyn_lds, s>>>(a);
-        LF_HIP(hipGetLastError());
-        if (L.n_heavy > 0) {
-            const int sw = kWG / plan->lpr;
-            const int fgrid = std::min((L.n_heavy + sw - 1) / sw, 1024);
-            ks.finalize<<<fgrid, kWG, 0, s>>>(plan->d_heavy + L.heavy_begin, L.n_heavy, a);
+    // One pass per feature window (all partitions inside), each on its own columns of B and C.
+    const size_t b_elem = plan->b_dtype == LF_DTYPE_BF16 ? 2 : 4;
+    const int ld = plan->feat * plan->windows;
+    for (int w = 0; w < plan->windows; ++w) {
+        for (int p = 0; p < plan->num_parts; ++p) {
+            const lf_spmm_plan::Launch& L = plan->launches[p];
+            if (L.n_groups == 0) continue;
+            LaunchArgs a{};
+            a.groups = plan->d_groups + L.group_begin;
+            a.n_groups = L.n_groups;
+            a.accumulate = p > 0 ? 1 : 0;
+            a.feat = plan->feat;
+            a.ldb = a.ldc = ld;
+            a.B = (const char*)d_B + (size_t)w * plan->feat * b_elem;
+            a.C = d_C + (size_t)w * plan->feat;
+            a.partials = plan->d_partials;
+            ks.tiles<<<L.grid, kWG, L.dyn_lds, s>>>(a);
             LF_HIP(hipGetLastError());
+            if (L.n_heavy > 0) {
+                const int sw = kWG / plan->lpr;
+                const int fgrid = std::min((L.n_heavy + sw - 1) / sw, 1024);
+                ks.finalize<<<fgrid, kWG, 0, s>>>(plan->d_heavy + L.heavy_begin, L.n_heavy, a);
+                LF_HIP(hipGetLastError());
+            }
         }
     }
+    return LF_OK;
+}
+
+int lf_spmm_set_windows(lf_spmm_plan* plan, int32_t n_windows) {
+    LF_REQUIRE(plan, LF_ERR_INVALID, "plan is null");
+    LF_REQUIRE(n_windows >= 1 && (int64_t)n_windows * plan->feat <= (1 << 20), LF_ERR_INVALID,
+               "bad number of feature windows (%d)", n_windows);
+    plan->windows = n_windows;
     return LF_OK;
 }
 
@@ -1269,6 +1287,7 @@ int lf_csr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const float* 
     if (int rc = select_kernels(lpr, ch, b_dtype, &ks)) return rc;
     LaunchArgs a{};
     a.feat = feat_size;
+    a.ldb = a.ldc = feat_size;
     a.B = d_B;
     a.C = d_C;
     const int sw = kWG / lpr;

@@ -66,7 +66,7 @@ def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="
 
     table = {k: [] for k in ("name", "format", "feat_size", "num_parts", "time_select(s)",
                              "time_num_parts(s)", "time_bucket(s)", "time_exe_our(ms)",
-                             "time_compose(ms)", "GFLOP/s", "bucket_config")}
+                             "time_compose(ms)", "GFLOP/s", "feature_windows", "bucket_config")}
     for g in matrices:
         print(f"\nGo to name {g.name} ...")
         fa._device_csr(g)          # the matrix goes to the GPU when it is loaded, before any timed step
@@ -81,20 +81,20 @@ def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="
                        "time_select(s)": time_select, "time_num_parts(s)": 0, "time_bucket(s)": 0,
                        "time_exe_our(ms)": exe_time, "time_compose(ms)": float("nan"),
                        "GFLOP/s": 2.0 * g.num_edges() * feat / (exe_time * 1e-3) / 1e9 if exe_time > 0 else 0.0,
-                       "bucket_config": ""}
+                       "feature_windows": 1, "bucket_config": ""}
                 for k, v in row.items():
                     table[k].append(v)
             continue
         for feat in feat_sizes:
             t0 = time.perf_counter()
             if num_parts is None:
-                parts = fa.choose_num_partitions(g, feat, cost_model=cost_model)
+                parts, windows = fa.choose_launch_shape(g, feat, cost_model=cost_model)
             elif callable(num_parts):
-                parts = int(num_parts(g, feat))
+                parts, windows = int(num_parts(g, feat)), 1
             else:
-                parts = int(num_parts)
+                parts, windows = int(num_parts), 1
             time_parts = time.perf_counter() - t0
-            print(f"name: {g.name} num_parts: {parts} time(s): {time_parts}")
+            print(f"name: {g.name} num_parts: {parts} feature_windows: {windows} time(s): {time_parts}")
 
             print("Configuring ...", flush=True)
             t0 = time.perf_counter()                                   # proc05:153-157
@@ -114,7 +114,8 @@ def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="
                 exe_time = fa.bench_hyb_with_config(g, x, y_ndarray, feat_size=feat, bucket_widths=bucket_config,
                                                     bucketing_format=hyb, coarsening_factor=2,
                                                     num_col_parts=parts, use_implicit_unroll=True,
-                                                    check_correctness=check_correctness)
+                                                    check_correctness=check_correctness,
+                                                    feature_windows=windows)
                 print(f"name: {g.name} format: {fmt_name} feat_size: {feat} num_partitions: {parts} "
                       f"cost_model_config: {cfg} bucket_config: {bucket_config} exe_time: {exe_time}", flush=True)
             except Exception as e:                                     # proc05:178-180
@@ -124,6 +125,7 @@ def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="
             table["format"].append(fmt_name)
             table["feat_size"].append(feat)
             table["num_parts"].append(parts)
+            table["feature_windows"].append(windows)
             table["time_select(s)"].append(time_select)
             table["time_num_parts(s)"].append(time_parts)
             table["time_bucket(s)"].append(time_bucket)

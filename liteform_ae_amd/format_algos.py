@@ -35,7 +35,7 @@ from .format_matrix_market import MTX, Bucket  # noqa: F401  (re-exported like t
 __all__ = ["build_hyb_format", "bench_hyb_with_config", "search_bucket_config",
            "CostModelSettings", "bench_bsrmm", "bench_naive", "spmm_bsr",
            "build_hyb_format_device", "HybFormat", "HybSpMM", "spmm_hyb", "spmm_csr",
-           "guess_num_partitions", "choose_num_partitions", "matrix_features_device"]
+           "guess_num_partitions", "choose_num_partitions", "choose_launch_shape", "matrix_features_device"]
 
 WIDTH_LIMIT = 1024   # format_algos.py:821
 
@@ -337,11 +337,17 @@ def build_hyb_format(g, bucket_widths):
 
 # --------------------------------------------------------------------------- SpMM
 class HybSpMM:
-    """Kernel plan for C = A_hyb . B on the current device (wraps lf_spmm_plan)."""
+    """Kernel plan for C = A_hyb . B on the current device (wraps lf_spmm_plan).
+
+    ``windows`` > 1 computes the product in that many passes over ``feat_size // windows``
+    features each (lf_spmm_set_windows): same result up to the summation order of the
+    cooperatively reduced rows, and faster when B is much larger than the memory-side cache."""
 
     def __init__(self, fmt_or_slabs, feat_size: int, b_dtype: str = "f32", num_rows=None, num_cols=None,
-                 bucket_widths=None):
+                 bucket_widths=None, windows: int = 1):
         torch = _torch()
+        if windows < 1 or feat_size % windows:
+            raise ValueError(f"feat_size {feat_size} is not a multiple of windows {windows}")
         lib = _lib.load()
         self._lib = lib
         self._keep = []
@@ -376,12 +382,17 @@ class HybSpMM:
         self.b_dtype = b_dtype
         self.num_rows, self.num_cols = int(num_rows), int(num_cols)
         dt = {"f32": _lib.LF_DTYPE_F32, "bf16": _lib.LF_DTYPE_BF16}[b_dtype]
+        self.windows = int(windows)
         _lib.check(lib.lf_spmm_create(C.byref(self.handle), descs, nb, P, self.num_rows, self.num_cols,
-                                      self.feat_size, dt, _stream()))
+                                      self.feat_size // self.windows, dt, _stream()))
+        if self.windows > 1:
+            _lib.check(lib.lf_spmm_set_windows(self.handle, self.windows))
         info = np.zeros(8, dtype=np.int64)
         _lib.check(lib.lf_spmm_info(self.handle, _lib.np_ptr(info, C.c_int64)))
         self.info = dict(zip(["tiles", "grid", "launches", "lds_bytes", "heavy_rows", "partial_rows",
                               "cleared_rows", "occupancy"], info.tolist()))
+        self.info["launches"] *= self.windows
+        self.info["windows"] = self.windows
 
     def _check_operands(self, B, Cout):
         torch = _torch()
@@ -462,9 +473,10 @@ def _timing_params():
 
 def bench_hyb_with_config(g, x, y_ndarray, feat_size=128, bucket_widths=[], bucketing_format=[],
                           coarsening_factor=2, num_col_parts=1, use_implicit_unroll=False,
-                          check_correctness=False):
+                          check_correctness=False, feature_windows=1):
     """Build and time the fused hyb SpMM kernel; returns the mean kernel time in ms
-    (format_algos.py:388-605).
+    (format_algos.py:388-605).  ``feature_windows`` (not in the reference) computes the
+    product in that many passes over the features, see ``HybSpMM``.
 
     ``bucketing_format`` is what build_hyb_format returned - then, as in the reference, the
     mask is used as A's values (format_algos.py:568-570) - or a ``HybFormat`` from
@@ -475,10 +487,10 @@ def bench_hyb_with_config(g, x, y_ndarray, feat_size=128, bucket_widths=[], buck
     num_rows = g.num_src_nodes()
     num_cols = g.num_dst_nodes()
     if isinstance(bucketing_format, HybFormat):
-        plan = HybSpMM(bucketing_format, feat_size, "f32")
+        plan = HybSpMM(bucketing_format, feat_size, "f32", windows=feature_windows)
     else:
         plan = HybSpMM(bucketing_format, feat_size, "f32", num_rows=num_rows, num_cols=num_cols,
-                       bucket_widths=[list(ws) for ws in bucket_widths][:num_col_parts])
+                       bucket_widths=[list(ws) for ws in bucket_widths][:num_col_parts], windows=feature_windows)
     try:
         xb = x.numpy() if hasattr(x, "numpy") else np.asarray(x)
         B = torch.from_numpy(np.ascontiguousarray(xb.reshape(num_cols, feat_size), dtype=np.float32)).cuda()
@@ -640,14 +652,25 @@ def guess_num_partitions(g, feat_size: int, b_dtype: str = "f32") -> int:
     return int(min(4, max(1, round(b_bytes / (2.5 * MALL_BYTES)))))
 
 
-def choose_num_partitions(g, feat_size: int, b_dtype: str = "f32", candidates: Sequence[int] = (1, 2, 3, 4),
-                          cost_model: str = "gfx950", runs: int = 5, return_timings: bool = False):
-    """Column-partition count by measurement: composes the format for every candidate and
-    times the fused kernel (a few runs each); returns the smallest count whose time is within
-    2 % of the fastest.  Takes the place of the
-    reference's partition predictor (proc05.spmm.end-to-end.py:142)."""
+def _window_candidates(feat_size: int, b_dtype: str) -> List[int]:
+    """Feature-window counts worth timing: windows of at least 64 features (32-feature
+    passes lost on every matrix measured) that the kernels support."""
+    step = 64 if b_dtype == "bf16" else 32
+    return [w for w in (1, 2, 4, 8) if feat_size % w == 0 and feat_size // w >= 64 and (feat_size // w) % step == 0] or [1]
+
+
+def choose_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Sequence[int] = (1, 2, 3, 4),
+                        windows: Sequence[int] = None, cost_model: str = "gfx950", runs: int = 5,
+                        return_timings: bool = False):
+    """Column-partition count and feature-window count by measurement: composes the format
+    for every candidate partition count, times the fused kernel for every window count (a
+    few runs each) and returns the pair (partitions, windows) with the fewest launches among
+    those within 2 % of the fastest.  Takes the place of the reference's partition predictor
+    (proc05.spmm.end-to-end.py:142); feature windows have no counterpart there."""
     torch = _torch()
     want = torch.float32 if b_dtype == "f32" else torch.bfloat16
+    if windows is None:
+        windows = _window_candidates(feat_size, b_dtype)
     # random operand: constant data lets the GPU clock higher and flatters every candidate
     B = (torch.rand((g.num_dst_nodes(), feat_size), dtype=torch.float32, device="cuda") - 0.5).to(want)
     Cout = torch.empty((g.num_src_nodes(), feat_size), dtype=torch.float32, device="cuda")
@@ -658,16 +681,27 @@ def choose_num_partitions(g, feat_size: int, b_dtype: str = "f32", candidates: S
         except ValueError:
             continue                      # a partition with a single nonzero: not a usable split
         fmt = build_hyb_format_device(g, cfg)
-        plan = HybSpMM(fmt, feat_size, b_dtype)
-        try:
-            timings[p] = float(np.median(plan.time_ms(B, Cout, warmup=2, repeat=runs)))
-        finally:
-            plan.close()
+        for w in windows:
+            plan = HybSpMM(fmt, feat_size, b_dtype, windows=w)
+            try:
+                timings[(p, w)] = float(np.median(plan.time_ms(B, Cout, warmup=2, repeat=runs)))
+            finally:
+                plan.close()
         del fmt
     if not timings:
         raise ValueError("no candidate partition count is usable for this matrix")
-    # the smallest count within 2 % of the fastest: fewer partitions mean fewer launches and
-    # less memory, and differences below that are run-to-run noise
+    # fewest launches within 2 % of the fastest: fewer partitions mean less memory and fewer
+    # passes over C, and differences below that are run-to-run noise
     fastest = min(timings.values())
-    best = min(p for p, t in timings.items() if t <= 1.02 * fastest)
+    best = min((k for k, t in timings.items() if t <= 1.02 * fastest), key=lambda k: (k[0] * k[1], k[0]))
     return (best, timings) if return_timings else best
+
+
+def choose_num_partitions(g, feat_size: int, b_dtype: str = "f32", candidates: Sequence[int] = (1, 2, 3, 4),
+                          cost_model: str = "gfx950", runs: int = 5, return_timings: bool = False):
+    """Column-partition count by measurement for a single pass over the features
+    (choose_launch_shape with one window)."""
+    best, timings = choose_launch_shape(g, feat_size, b_dtype, candidates, windows=(1,), cost_model=cost_model,
+                                        runs=runs, return_timings=True)
+    flat = {p: t for (p, _), t in timings.items()}
+    return (best[0], flat) if return_timings else best[0]

@@ -259,3 +259,41 @@ def test_partition_chooser_and_driver_table(fa, torch):
     assert list(df.columns[:8]) == ["name", "format", "feat_size", "num_parts", "time_select(s)",
                                     "time_num_parts(s)", "time_bucket(s)", "time_exe_our(ms)"]
     assert len(df) == 2 and (df["format"] == "CELL").all() and np.isfinite(df["time_exe_our(ms)"]).all()
+
+
+@pytest.mark.parametrize("feat,b_dtype,windows", [(128, "f32", 2), (256, "f32", 4), (512, "f32", 2), (256, "bf16", 2),
+                                                  (1024, "bf16", 4), (96, "f32", 3)])
+def test_feature_windows_match_single_pass(fa, torch, feat, b_dtype, windows):
+    """The product in several passes over feature windows: within tolerance of the oracle and
+    equal to the single-pass result on rows that are summed slot by slot in one ELL row (split
+    and cooperatively reduced rows are summed in pieces whose size follows the lane count)."""
+    rng = np.random.default_rng(800 + feat)
+    g = skewed_matrix(rng, 2000, 2600, mean_deg=12, heavy_rows=3, heavy_len=2400)
+    nr, nc = g.coo_mtx.shape
+    B = rng.uniform(-1, 1, size=(nc, feat)).astype(np.float32)
+    Bd = torch.from_numpy(B).cuda()
+    if b_dtype == "bf16":
+        Bd = Bd.to(torch.bfloat16)
+        B = Bd.to(torch.float32).cpu().numpy()
+    indptr, indices, data = g.adj_tensors("csr")
+    data = np.asarray(data, dtype=np.float32)
+    ref = O.spmm_csr_f64(indptr, indices, data, (nr, nc), B)
+    bound = O.spmm_abs_bound(indptr, indices, data, (nr, nc), B)
+    for widths in ([[1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024]], [[4, 32]], [[2, 16], [8, 64]]):
+        fmt = fa.build_hyb_format_device(g, widths)
+        one = fa.HybSpMM(fmt, feat, b_dtype)
+        many = fa.HybSpMM(fmt, feat, b_dtype, windows=windows)
+        assert many.info["windows"] == windows and many.info["launches"] == windows * one.info["launches"]
+        C1 = one.run(Bd).cpu().numpy()
+        Cw = many.run(Bd).cpu().numpy()
+        Cw2 = torch.full((nr, feat), 7.0, device="cuda")          # stale output is overwritten
+        many.run(Bd, Cw2)
+        one.close()
+        many.close()
+        np.testing.assert_array_equal(Cw, Cw2.cpu().numpy())
+        assert (np.abs(Cw.astype(np.float64) - ref) <= TOL * bound).all()
+        if len(widths[0]) == 11:          # every width present: a row up to 128 entries is one ELL row,
+            light = np.diff(indptr) <= 128        # summed slot by slot whatever the lane count
+            np.testing.assert_array_equal(Cw[light], C1[light])
+    with pytest.raises(ValueError):
+        fa.HybSpMM(fmt, feat, b_dtype, windows=7)
