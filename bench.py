@@ -44,13 +44,15 @@ def gather_bytes(nnz, rows, feat, b_bytes):
     return nnz * 8 + (rows + 1) * 4 + nnz * feat * b_bytes + rows * feat * 4
 
 
-# L2 <-> fabric bytes per step (all launches of a step) from rocprofv3 --pmc FETCH_SIZE and
+# L2 <-> fabric bytes per step (all launches of a step; /W2 = two feature windows) from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE, FETCH_SIZE scaled by 2.000 as calibrated on a 1 GiB copy in the same runs;
 # source: profiles/spmm_partition_kernel.cfg3_N128.md
 MEASURED_TRAFFIC = {
     "cfg3/N128/P1": 44157630417,
     "cfg3/N128/P2": 46512630501,
     "cfg3/N128/P3": 48665180588,
+    "cfg3/N128/P1/W2": 45234112102,
+    "cfg3/N128/P2/W2": 47336937882,
 }
 
 
