@@ -26,7 +26,9 @@ def test_operations_raise_without_gpu():
                  lambda: fa.build_hyb_format(g, [[1, 2]]),
                  lambda: fa.build_hyb_format_device(g, [[1, 2]]),
                  lambda: fa.bench_naive(g, np.ones((2, 32), np.float32), None, feat_size=32),
-                 lambda: fa.choose_num_partitions(g, 32)):
+                 lambda: fa.choose_num_partitions(g, 32),
+                 lambda: fa.choose_launch_shape(g, 128),
+                 lambda: fa.matrix_features_device(g)):
         with pytest.raises(RuntimeError, match="no CPU fallback"):
             call()
 
