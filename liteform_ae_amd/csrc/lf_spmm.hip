@@ -28,6 +28,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -663,6 +664,275 @@ spmm_finalize_kernel(const HeavyRow* __restrict__ heavy, int n_heavy, LaunchArgs
     }
 }
 
+// ------------------------------------------------------------------------------------
+// Row groups.  In a banded, stencil or block-structured matrix consecutive rows hold mostly
+// the same columns; a bucket of such rows is rewritten at plan time as groups of four
+// consecutive ELL rows with the union of their columns ("merged entries": column, four
+// values, a 4-bit presence mask), and one gather of a B row then feeds up to four output
+// rows.  The 27-point stencil needs 54 gathers per four rows instead of 4 x 28.  Only
+// buckets whose merged entries are well below their slots take this path (measured at plan
+// time); a matrix without shared columns never does.  Separate kernel, so that its registers
+// (four accumulators) do not weigh on the main one.
+constexpr int kGroupRows = 4;
+constexpr int kMergedCap = 384;        // merged entries staged per workgroup at most
+constexpr int kMergedTileGroups = 64;  // row groups per tile at most
+constexpr long long kRowGroupMinRows = 4096;   // smaller buckets are not worth the analysis
+constexpr int kRowGroupSample = 4096;          // the decision looks at about this many groups of a bucket first
+constexpr int kRowGroupMaxPercent = 70;        // merged entries / plain gathers at most, in percent
+constexpr int kRowGroupSampleEntries = 24;     // merged entries of a group that the sampling pass looks at
+
+struct MergedBucket {
+    long long n_groups;        // row groups
+    long long n_rows;          // ELL rows of the bucket (the last group may hold fewer than four)
+    long long n_tiles;
+    int groups_per_tile;
+    int pad_;
+    const int32_t* rows;       // [n_rows] source rows of the bucket
+    const int32_t* goff;       // [n_groups + 1] first merged entry of each group
+    const int32_t* ecol;       // [entries]
+    const float4* eval;        // [entries] the four rows' values, 0 where a row lacks the column
+    const uint8_t* emask;      // [entries] bit r: row r of the group holds the column
+};
+
+// Merges the (ascending) column lists of the rows of group g; calls emit(col, vals[4], mask)
+// per merged entry when kEmit, and returns the number of merged entries.
+template <bool kEmit, typename Emit>
+__device__ __forceinline__ int merge_group(const int32_t* __restrict__ cols, const float* __restrict__ vals,
+                                           const int32_t* __restrict__ meta, long long g, long long n_rows,
+                                           int log_w, Emit emit, int max_entries = 0x7FFFFFFF,
+                                           int* consumed = nullptr) {
+    // Four columns (and values) of every row are held in registers and refilled with one
+    // 16-byte load: a row starts at a multiple of its width (>= 8 slots), so the loads are
+    // aligned, and the chain of dependent loads is a quarter as long.
+    int len[kGroupRows], pos[kGroupRows];
+    long long base[kGroupRows];
+    int4 cbuf[kGroupRows];
+    float4 vbuf[kGroupRows];
+#pragma unroll
+    for (int r = 0; r < kGroupRows; ++r) {
+        const long long e = g * kGroupRows + r;
+        len[r] = e < n_rows ? (meta[e] & (int)kMetaLenMask) : 0;
+        base[r] = e << log_w;
+        pos[r] = 0;
+        cbuf[r] = make_int4(0, 0, 0, 0);
+        vbuf[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (len[r] > 0) {
+            cbuf[r] = *reinterpret_cast<const int4*>(cols + base[r]);
+            if (kEmit) vbuf[r] = *reinterpret_cast<const float4*>(vals + base[r]);
+        }
+    }
+    auto pick = [](const int4& q, int i) { return i == 0 ? q.x : i == 1 ? q.y : i == 2 ? q.z : q.w; };
+    auto pickf = [](const float4& q, int i) { return i == 0 ? q.x : i == 1 ? q.y : i == 2 ? q.z : q.w; };
+    int m = 0;
+    for (;;) {
+        int head[kGroupRows];
+        int cmin = 0x7FFFFFFF;
+#pragma unroll
+        for (int r = 0; r < kGroupRows; ++r) {
+            head[r] = pos[r] < len[r] ? pick(cbuf[r], pos[r] & 3) : 0x7FFFFFFF;
+            cmin = min(cmin, head[r]);
+        }
+        if (cmin == 0x7FFFFFFF) break;
+        float v[kGroupRows];
+        uint32_t mask = 0;
+#pragma unroll
+        for (int r = 0; r < kGroupRows; ++r) {
+            v[r] = 0.f;
+            if (head[r] == cmin) {
+                if (kEmit) v[r] = pickf(vbuf[r], pos[r] & 3);
+                mask |= 1u << r;
+                ++pos[r];
+                if ((pos[r] & 3) == 0 && pos[r] < len[r]) {
+                    cbuf[r] = *reinterpret_cast<const int4*>(cols + base[r] + pos[r]);
+                    if (kEmit) vbuf[r] = *reinterpret_cast<const float4*>(vals + base[r] + pos[r]);
+                }
+            }
+        }
+        if (kEmit) emit(m, cmin, v, mask);
+        if (++m >= max_entries) break;
+    }
+    if (consumed) *consumed = pos[0] + pos[1] + pos[2] + pos[3];
+    return m;
+}
+
+// One candidate bucket of the row-group analysis.
+struct RowGroupCand {
+    const int32_t* cols;
+    const int32_t* meta;
+    long long n_rows;
+    long long n_groups;
+    int32_t* m_out;            // merged length of every group, or null
+    int log_w;
+    int stride;                // > 1: only every stride-th group is looked at (sampling)
+};
+
+// counters[3 * cand + ...]: [0] merged entries, [1] gathers of the plain path (row lengths
+// rounded up to the unroll; when sampling, the slots that the merged entries consumed),
+// [2] longest group.  blockIdx.y is the candidate.
+__global__ void __launch_bounds__(256)
+rowgroup_count_kernel(const RowGroupCand* __restrict__ cands, unsigned long long* __restrict__ counters) {
+    const RowGroupCand cd = cands[blockIdx.y];
+    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long g = t * cd.stride;
+    int m = 0, plain = 0;
+    if (g < cd.n_groups) {
+        if (cd.stride > 1) {
+            // sampling: the first merged entries of the group against the slots they consume
+            m = merge_group<false>(cd.cols, nullptr, cd.meta, g, cd.n_rows, cd.log_w,
+                                   [](int, int, const float*, uint32_t) {}, kRowGroupSampleEntries, &plain);
+        } else {
+            m = merge_group<false>(cd.cols, nullptr, cd.meta, g, cd.n_rows, cd.log_w, [](int, int, const float*, uint32_t) {});
+            for (int r = 0; r < kGroupRows; ++r) {
+                const long long e = g * kGroupRows + r;
+                if (e < cd.n_rows) plain += ((cd.meta[e] & (int)kMetaLenMask) + kUnroll - 1) / kUnroll * kUnroll;
+            }
+        }
+        if (cd.m_out) cd.m_out[g] = m;
+    }
+    int sm = m, sp = plain, mx = m;
+    for (int d = 32; d > 0; d >>= 1) {
+        sm += __shfl_xor(sm, d);
+        sp += __shfl_xor(sp, d);
+        mx = max(mx, __shfl_xor(mx, d));
+    }
+    if ((threadIdx.x & 63) == 0 && sp > 0) {
+        unsigned long long* c = counters + 3 * blockIdx.y;
+        atomicAdd(&c[0], (unsigned long long)sm);
+        atomicAdd(&c[1], (unsigned long long)sp);
+        atomicMax(&c[2], (unsigned long long)mx);
+    }
+}
+
+// goff[g] = exclusive prefix of m[g] (in place is not possible: goff has one more entry);
+// single workgroup, the arrays are a few hundred thousand entries.
+__global__ void __launch_bounds__(1024)
+rowgroup_scan_kernel(const int32_t* __restrict__ m, long long n_groups, int32_t* __restrict__ goff) {
+    __shared__ int s_wave[16];
+    __shared__ int s_carry;
+    if (threadIdx.x == 0) s_carry = 0;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (long long base = 0; base < n_groups; base += 1024) {
+        const long long i = base + threadIdx.x;
+        const int x = i < n_groups ? m[i] : 0;
+        int incl = x;
+        for (int d = 1; d < 64; d <<= 1) {
+            const int y = __shfl_up(incl, d);
+            if (lane >= d) incl += y;
+        }
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        int off = s_carry;
+        for (int w = 0; w < wave; ++w) off += s_wave[w];
+        if (i < n_groups) goff[i] = off + incl - x;
+        __syncthreads();
+        if (threadIdx.x == 1023) s_carry = off + incl;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) goff[n_groups] = s_carry;
+}
+
+__global__ void __launch_bounds__(256)
+rowgroup_fill_kernel(const int32_t* __restrict__ cols, const float* __restrict__ vals,
+                     const int32_t* __restrict__ meta, long long n_rows, int log_w, long long n_groups,
+                     const int32_t* __restrict__ goff, int32_t* __restrict__ ecol, float4* __restrict__ eval,
+                     uint8_t* __restrict__ emask) {
+    const long long g = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= n_groups) return;
+    const long long at = goff[g];
+    merge_group<true>(cols, vals, meta, g, n_rows, log_w, [&](int j, int c, const float* v, uint32_t mask) {
+        ecol[at + j] = c;
+        eval[at + j] = make_float4(v[0], v[1], v[2], v[3]);
+        emask[at + j] = (uint8_t)mask;
+    });
+}
+
+// One workgroup per tile of row groups, XCD-aware like the main kernel.  CH == 1 only.
+template <int LPR, typename BT>
+__global__ void __launch_bounds__(kWG)
+spmm_rowgroup_kernel(const MergedBucket* __restrict__ buckets, int n_buckets, LaunchArgs a) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int SW = kWG / LPR;
+    constexpr int U = VEC == 4 ? 8 : 4;          // gathers in flight per sub-wave
+    __shared__ float4 s_val[kMergedCap];
+    __shared__ int s_col[kMergedCap];
+    __shared__ int s_goff[kMergedTileGroups + 1];
+    __shared__ uint8_t s_msk[kMergedCap];
+
+    const int xcd = blockIdx.x % kXcds;
+    long long v = blockIdx.x / kXcds;
+    for (int bi = 0; bi < n_buckets; ++bi) {
+        const MergedBucket& b = buckets[bi];
+        const long long lo = b.n_tiles * xcd / kXcds;
+        const long long hi = b.n_tiles * (xcd + 1) / kXcds;
+        if (v >= hi - lo) { v -= hi - lo; continue; }
+        const long long g0 = (lo + v) * b.groups_per_tile;
+        const int n = (int)min((long long)b.groups_per_tile, b.n_groups - g0);
+        const int tid = threadIdx.x;
+        for (int i = tid; i <= n; i += kWG) s_goff[i] = b.goff[g0 + i];
+        __syncthreads();
+        const int base = s_goff[0];
+        const int n_entries = s_goff[n] - base;            // <= kMergedCap by the choice of groups_per_tile
+        for (int i = tid; i < n_entries; i += kWG) {
+            s_col[i] = b.ecol[base + i];
+            s_val[i] = b.eval[base + i];
+            s_msk[i] = b.emask[base + i];
+        }
+        __syncthreads();
+        const int sw = tid / LPR, sl = tid % LPR;
+        const Lane<LPR, 1, VEC> ln(sl, a.feat, a.ldb, a.ldc);
+        for (int gi = sw; gi < n; gi += SW) {
+            const int e0 = s_goff[gi] - base;
+            const int m = s_goff[gi + 1] - s_goff[gi];
+            Acc<1, VEC> acc[kGroupRows];
+#pragma unroll
+            for (int r = 0; r < kGroupRows; ++r) acc[r].clear();
+            for (int j = 0; j < m; j += U) {
+                int c[U];
+                float4 w[U];
+                uint32_t k[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const bool in = j + u < m;
+                    const int idx = e0 + (in ? j + u : 0);   // past the end: the first column again, nothing added
+                    c[u] = s_col[idx];
+                    w[u] = in ? s_val[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    k[u] = in ? s_msk[idx] : 0u;
+                }
+                float x[U][VEC];
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    Dense<BT>::load(a.B, (size_t)(uint32_t)c[u] * (size_t)ln.ldb + ln.f[0], x[u]);
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const float wr[kGroupRows] = {w[u].x, w[u].y, w[u].z, w[u].w};
+#pragma unroll
+                    for (int r = 0; r < kGroupRows; ++r) {
+                        if constexpr (LPR == 64) {
+                            // one group per wavefront: rows without the column are skipped outright
+                            if (__builtin_amdgcn_readfirstlane(k[u]) & (1u << r)) {
+#pragma unroll
+                                for (int i = 0; i < VEC; ++i) acc[r].v[0][i] = fmaf(wr[r], x[u][i], acc[r].v[0][i]);
+                            }
+                        } else {
+                            // several groups per wavefront: the value is 0 where the row lacks the
+                            // column (like a padded slot, this adds 0 * B: only non-finite B differs)
+#pragma unroll
+                            for (int i = 0; i < VEC; ++i) acc[r].v[0][i] = fmaf(wr[r], x[u][i], acc[r].v[0][i]);
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < kGroupRows; ++r) {
+                const long long e = (g0 + gi) * kGroupRows + r;
+                if (e < b.n_rows) store_row<LPR, 1, VEC>(a.C, b.rows[e], ln, acc[r], a.accumulate);
+            }
+        }
+        return;
+    }
+}
+
 // Row-parallel CSR product: one sub-wave per row, entries streamed by shuffle.
 template <int LPR, int CH, typename BT>
 __global__ void __launch_bounds__(kWG)
@@ -840,10 +1110,12 @@ struct lf_spmm_plan {
     struct Launch {
         int group_begin = 0, n_groups = 0, grid = 0;
         int dyn_lds = 0;             // bytes of dynamic LDS (balanced segment tiles)
+        int merged_begin = 0, n_merged = 0, merged_grid = 0;   // row-group buckets of this partition
         long long tiles = 0;
         int heavy_begin = 0, n_heavy = 0;
     };
     std::vector<Launch> launches;
+    MergedBucket* d_merged = nullptr;   // row-group buckets, grouped by partition
     std::vector<void*> owned;        // device allocations released by destroy
     Group* d_groups = nullptr;
     HeavyRow* d_heavy = nullptr;
@@ -867,13 +1139,20 @@ using KernelFn = void (*)(LaunchArgs);
 using FinalFn = void (*)(const HeavyRow*, int, LaunchArgs);
 using CsrFn = void (*)(const int32_t*, const int32_t*, const float*, long long, LaunchArgs);
 
+using RowGroupFn = void (*)(const MergedBucket*, int, LaunchArgs);
+
 struct KernelSet {
     KernelFn tiles = nullptr;
     FinalFn finalize = nullptr;
     CsrFn csr = nullptr;
+    RowGroupFn rowgroup = nullptr;   // one 16-byte chunk per lane only
 };
 
 template <int LPR, int CH> void pick_kernels(int dtype, KernelSet* k) {
+    if constexpr (CH == 1) {
+        if (dtype == LF_DTYPE_BF16) k->rowgroup = spmm_rowgroup_kernel<LPR, bf16_t>;
+        else k->rowgroup = spmm_rowgroup_kernel<LPR, float>;
+    }
     if (dtype == LF_DTYPE_BF16) {
         k->tiles = spmm_partition_kernel<LPR, CH, bf16_t>;
         k->finalize = spmm_finalize_kernel<LPR, CH, bf16_t>;
@@ -1104,6 +1383,94 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         LF_TRY_HIP(hipGetLastError());
     }
 
+    // ---- row groups: buckets whose consecutive rows share most of their columns
+    std::vector<MergedBucket> merged;                      // in bucket (hence partition) order
+    std::vector<int> merged_of((size_t)num_buckets, -1);
+    {
+        const char* env = getenv("LF_ROW_GROUPS");
+        std::vector<int> cand;
+        for (int k = 0; k < num_buckets && ch == 1 && !(env && env[0] == '0'); ++k) {
+            const lf_bucket_desc& b = h_buckets[k];
+            if (b.num_ell_rows >= kRowGroupMinRows && b.width >= kUnroll && b.width <= 64 && !is_multi[k]) cand.push_back(k);
+        }
+        unsigned long long* d_rg = nullptr;                // three counters per candidate
+        std::vector<unsigned long long> h_rg(cand.size() * 3, 0);
+        RowGroupCand* d_cands = nullptr;
+        auto count_pass = [&](const std::vector<int>& which, bool sample, std::vector<int32_t*>* m_arrays) -> int {
+            std::vector<RowGroupCand> h_cands(which.size());
+            long long most = 1;
+            for (size_t i = 0; i < which.size(); ++i) {
+                const lf_bucket_desc& b = h_buckets[which[i]];
+                RowGroupCand& c = h_cands[i];
+                c.cols = b.d_cols;
+                c.meta = meta[which[i]];
+                c.n_rows = b.num_ell_rows;
+                c.n_groups = lf::ceil_div(b.num_ell_rows, kGroupRows);
+                c.m_out = m_arrays ? (*m_arrays)[i] : nullptr;
+                c.log_w = lf::ilog2(b.width);
+                c.stride = sample ? (int)std::max<long long>(1, c.n_groups / kRowGroupSample) : 1;
+                most = std::max<long long>(most, lf::ceil_div(c.n_groups, c.stride));
+            }
+            LF_HIP(hipMemsetAsync(d_rg, 0, cand.size() * 24, s));
+            LF_HIP(hipMemcpyAsync(d_cands, h_cands.data(), h_cands.size() * sizeof(RowGroupCand), hipMemcpyHostToDevice, s));
+            rowgroup_count_kernel<<<dim3((unsigned)lf::ceil_div(most, 256), (unsigned)which.size()), 256, 0, s>>>(d_cands, d_rg);
+            LF_HIP(hipGetLastError());
+            LF_HIP(hipMemcpyAsync(h_rg.data(), d_rg, which.size() * 24, hipMemcpyDeviceToHost, s));
+            LF_HIP(hipStreamSynchronize(s));               // also keeps h_cands alive until the copy is done
+            return LF_OK;
+        };
+        if (!cand.empty()) {
+            LF_TRY(dev_alloc(plan, &d_rg, cand.size() * 3));
+            LF_TRY(dev_alloc(plan, &d_cands, cand.size()));
+            LF_TRY(count_pass(cand, true, nullptr));       // a sample of the groups decides
+            std::vector<int> chosen;
+            for (size_t i = 0; i < cand.size(); ++i)
+                if (h_rg[3 * i + 1] > 0 && h_rg[3 * i] * 100 <= h_rg[3 * i + 1] * kRowGroupMaxPercent) chosen.push_back(cand[i]);
+            if (!chosen.empty()) {
+                std::vector<int32_t*> m_arrays(chosen.size(), nullptr);
+                for (size_t i = 0; i < chosen.size(); ++i)
+                    LF_TRY(dev_alloc(plan, &m_arrays[i], (size_t)lf::ceil_div(h_buckets[chosen[i]].num_ell_rows, kGroupRows)));
+                LF_TRY(count_pass(chosen, false, &m_arrays));
+                for (size_t i = 0; i < chosen.size(); ++i) {
+                    const int k = chosen[i];
+                    const lf_bucket_desc& b = h_buckets[k];
+                    const unsigned long long entries = h_rg[3 * i], plain = h_rg[3 * i + 1], longest = h_rg[3 * i + 2];
+                    if (entries == 0 || entries >= (1ull << 31) || longest > (unsigned long long)kMergedCap ||
+                        entries * 100 > plain * kRowGroupMaxPercent)
+                        continue;
+                    MergedBucket mb{};
+                    mb.n_rows = b.num_ell_rows;
+                    mb.n_groups = lf::ceil_div(b.num_ell_rows, kGroupRows);
+                    int32_t *goff = nullptr, *ecol = nullptr;
+                    float4* eval = nullptr;
+                    uint8_t* emask = nullptr;
+                    LF_TRY(dev_alloc(plan, &goff, (size_t)mb.n_groups + 1));
+                    LF_TRY(dev_alloc(plan, &ecol, (size_t)entries));
+                    LF_TRY(dev_alloc(plan, &eval, (size_t)entries));
+                    LF_TRY(dev_alloc(plan, &emask, (size_t)entries));
+                    rowgroup_scan_kernel<<<1, 1024, 0, s>>>(m_arrays[i], mb.n_groups, goff);
+                    LF_TRY_HIP(hipGetLastError());
+                    rowgroup_fill_kernel<<<(int)lf::ceil_div(mb.n_groups, 256), 256, 0, s>>>(
+                        b.d_cols, b.d_vals, meta[k], b.num_ell_rows, lf::ilog2(b.width), mb.n_groups, goff, ecol, eval, emask);
+                    LF_TRY_HIP(hipGetLastError());
+                    // tile: as many groups as the staging buffer surely holds, but enough tiles to spread
+                    long long per_tile = std::min<long long>(kMergedTileGroups, kMergedCap / (long long)longest);
+                    const long long spread = lf::ceil_div(mb.n_groups, (long long)4 * plan->num_cus);
+                    per_tile = std::max<long long>(1, std::min(per_tile, std::max<long long>(sw, spread)));
+                    mb.groups_per_tile = (int)per_tile;
+                    mb.n_tiles = lf::ceil_div(mb.n_groups, per_tile);
+                    mb.rows = b.d_rows;
+                    mb.goff = goff;
+                    mb.ecol = ecol;
+                    mb.eval = eval;
+                    mb.emask = emask;
+                    merged_of[k] = (int)merged.size();
+                    merged.push_back(mb);
+                }
+            }
+        }
+    }
+
     // ---- tile groups per launch: chunks first (longest), then buckets widest first, then clears
     std::vector<Group> groups;
     plan->launches.resize((size_t)num_parts);
@@ -1132,6 +1499,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         for (int k : mine) {
             const lf_bucket_desc& b = h_buckets[k];
             if (b.width > kCoopSlots) continue;            // every row of this bucket is a chunk
+            if (merged_of[k] >= 0) continue;               // served by the row-group kernel
             Group g{};
             g.log_w = lf::ilog2(b.width);
             const int fit = tile_slots(lpr) >> g.log_w;     // ELL rows whose slots fit the LDS tile
@@ -1172,6 +1540,23 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             groups.push_back(g);
         }
         L.n_groups = (int)groups.size() - L.group_begin;
+        L.merged_begin = -1;
+        for (int k : mine) {
+            if (merged_of[k] < 0) continue;
+            if (L.merged_begin < 0) L.merged_begin = merged_of[k];
+            ++L.n_merged;                                  // buckets of a partition are consecutive
+        }
+        if (L.n_merged > 0) {
+            long long longest_m = 0;
+            for (int x = 0; x < kXcds; ++x) {
+                long long len = 0;
+                for (int i = L.merged_begin; i < L.merged_begin + L.n_merged; ++i)
+                    len += merged[i].n_tiles * (x + 1) / kXcds - merged[i].n_tiles * x / kXcds;
+                longest_m = std::max(longest_m, len);
+            }
+            if (longest_m * kXcds >= (1ll << 31)) return bail(lf::fail(LF_ERR_UNSUPPORTED, "too many row-group tiles"));
+            L.merged_grid = (int)(longest_m * kXcds);
+        }
         // grid: 8 x the longest per-XCD tile list
         long long longest = 0;
         for (int x = 0; x < kXcds; ++x) {
@@ -1185,6 +1570,10 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             return bail(lf::fail(LF_ERR_UNSUPPORTED, "partition %d needs too many tiles", p));
         L.grid = (int)(longest * kXcds);
         total_tiles += L.tiles;
+    }
+    if (!merged.empty()) {
+        LF_TRY(dev_alloc(plan, &plan->d_merged, merged.size()));
+        LF_TRY_HIP(hipMemcpy(plan->d_merged, merged.data(), merged.size() * sizeof(MergedBucket), hipMemcpyHostToDevice));
     }
     if (!groups.empty()) {
         LF_TRY(dev_alloc(plan, &plan->d_groups, groups.size()));
@@ -1213,7 +1602,8 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     plan->info[4] = n_heavy_total;
     plan->info[5] = n_partials;
     plan->info[6] = n_zero;
-    plan->info[7] = occ;
+    (void)occ;
+    plan->info[7] = (int64_t)merged.size();
     LF_TRY_HIP(hipStreamSynchronize(s));     // the tables are complete: the plan may run on any stream
     *out_plan = plan;
     return LF_OK;
@@ -1241,7 +1631,7 @@ int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t str
     for (int w = 0; w < plan->windows; ++w) {
         for (int p = 0; p < plan->num_parts; ++p) {
             const lf_spmm_plan::Launch& L = plan->launches[p];
-            if (L.n_groups == 0) continue;
+            if (L.n_groups == 0 && L.n_merged == 0) continue;
             LaunchArgs a{};
             a.groups = plan->d_groups + L.group_begin;
             a.n_groups = L.n_groups;
@@ -1251,8 +1641,14 @@ int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t str
             a.B = (const char*)d_B + (size_t)w * plan->feat * b_elem;
             a.C = d_C + (size_t)w * plan->feat;
             a.partials = plan->d_partials;
-            ks.tiles<<<L.grid, kWG, L.dyn_lds, s>>>(a);
-            LF_HIP(hipGetLastError());
+            if (L.grid > 0) {
+                ks.tiles<<<L.grid, kWG, L.dyn_lds, s>>>(a);
+                LF_HIP(hipGetLastError());
+            }
+            if (L.n_merged > 0) {
+                ks.rowgroup<<<L.merged_grid, kWG, 0, s>>>(plan->d_merged + L.merged_begin, L.n_merged, a);
+                LF_HIP(hipGetLastError());
+            }
             if (L.n_heavy > 0) {
                 const int sw = kWG / plan->lpr;
                 const int fgrid = std::min((L.n_heavy + sw - 1) / sw, 1024);

@@ -390,7 +390,7 @@ class HybSpMM:
         info = np.zeros(8, dtype=np.int64)
         _lib.check(lib.lf_spmm_info(self.handle, _lib.np_ptr(info, C.c_int64)))
         self.info = dict(zip(["tiles", "grid", "launches", "lds_bytes", "heavy_rows", "partial_rows",
-                              "cleared_rows", "occupancy"], info.tolist()))
+                              "cleared_rows", "row_group_buckets"], info.tolist()))
         self.info["launches"] *= self.windows
         self.info["windows"] = self.windows
 

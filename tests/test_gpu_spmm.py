@@ -297,3 +297,36 @@ def test_feature_windows_match_single_pass(fa, torch, feat, b_dtype, windows):
             np.testing.assert_array_equal(Cw[light], C1[light])
     with pytest.raises(ValueError):
         fa.HybSpMM(fmt, feat, b_dtype, windows=7)
+
+
+def banded_matrix(rng, n, half_width, block=1):
+    """Rows hold the columns within half_width of the diagonal (clipped), in blocks of
+    `block` identical rows: consecutive rows share most (block > 1: all) of their columns."""
+    rows, cols = [], []
+    for r in range(n):
+        c0 = (r // block) * block
+        lo, hi = max(0, c0 - half_width), min(n, c0 + half_width + 1)
+        rows.append(np.full(hi - lo, r))
+        cols.append(np.arange(lo, hi))
+    rows, cols = np.concatenate(rows), np.concatenate(cols)
+    return MTX.from_coo(rows, cols, (n, n), data=rng.uniform(-1, 1, size=len(rows)).astype(np.float32))
+
+
+@pytest.mark.parametrize("feat,b_dtype", [(32, "f32"), (64, "f32"), (128, "f32"), (256, "f32"), (256, "bf16"),
+                                          (512, "bf16")])
+def test_rows_sharing_columns_are_served_in_groups(fa, torch, feat, b_dtype, monkeypatch):
+    """Banded and block-structured matrices: buckets whose consecutive rows share columns are
+    processed four rows at a time with shared gathers; a random matrix never is."""
+    rng = np.random.default_rng(900 + feat)
+    for g, widths in ((banded_matrix(rng, 9001, 10), [[8, 16, 32]]),          # 21 per row, last group partial
+                      (banded_matrix(rng, 6000, 7, block=4), [[16]]),          # 4 x 1 blocks: all columns shared
+                      (banded_matrix(rng, 10000, 12), [[16, 32], [8, 16]])):   # two partitions (second one adds)
+        _, info = check(fa, torch, g, widths, feat, b_dtype, seed=feat)
+        assert info["row_group_buckets"] >= 1, (widths, info)
+        monkeypatch.setenv("LF_ROW_GROUPS", "0")
+        _, info_off = check(fa, torch, g, widths, feat, b_dtype, seed=feat)
+        monkeypatch.delenv("LF_ROW_GROUPS")
+        assert info_off["row_group_buckets"] == 0
+    g = skewed_matrix(rng, 20000, 30000, mean_deg=20, heavy_rows=0)
+    _, info = check(fa, torch, g, [[8, 16, 32, 64]], feat, b_dtype, seed=feat)
+    assert info["row_group_buckets"] == 0
