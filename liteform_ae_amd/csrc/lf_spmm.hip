@@ -1543,8 +1543,8 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         L.merged_begin = -1;
         for (int k : mine) {
             if (merged_of[k] < 0) continue;
-            if (L.merged_begin < 0) L.merged_begin = merged_of[k];
-            ++L.n_merged;                                  // buckets of a partition are consecutive
+            if (L.merged_begin < 0 || merged_of[k] < L.merged_begin) L.merged_begin = merged_of[k];
+            ++L.n_merged;                                  // a partition's buckets are consecutive in `merged`
         }
         if (L.n_merged > 0) {
             long long longest_m = 0;

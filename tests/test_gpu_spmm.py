@@ -312,6 +312,18 @@ def banded_matrix(rng, n, half_width, block=1):
     return MTX.from_coo(rows, cols, (n, n), data=rng.uniform(-1, 1, size=len(rows)).astype(np.float32))
 
 
+def mixed_band_matrix(rng, n):
+    """Bands of 7, 13, 25 and 49 columns in turn, 2000 rows each: four buckets, all shared."""
+    rows, cols = [], []
+    for r in range(n):
+        half = (3, 6, 12, 24)[(r // 2000) % 4]
+        lo, hi = max(0, r - half), min(n, r + half + 1)
+        rows.append(np.full(hi - lo, r))
+        cols.append(np.arange(lo, hi))
+    rows, cols = np.concatenate(rows), np.concatenate(cols)
+    return MTX.from_coo(rows, cols, (n, n), data=rng.uniform(-1, 1, size=len(rows)).astype(np.float32))
+
+
 @pytest.mark.parametrize("feat,b_dtype", [(32, "f32"), (64, "f32"), (128, "f32"), (256, "f32"), (256, "bf16"),
                                           (512, "bf16")])
 def test_rows_sharing_columns_are_served_in_groups(fa, torch, feat, b_dtype, monkeypatch):
@@ -320,9 +332,10 @@ def test_rows_sharing_columns_are_served_in_groups(fa, torch, feat, b_dtype, mon
     rng = np.random.default_rng(900 + feat)
     for g, widths in ((banded_matrix(rng, 9001, 10), [[8, 16, 32]]),          # 21 per row, last group partial
                       (banded_matrix(rng, 6000, 7, block=4), [[16]]),          # 4 x 1 blocks: all columns shared
-                      (banded_matrix(rng, 10000, 12), [[16, 32], [8, 16]])):   # two partitions (second one adds)
+                      (banded_matrix(rng, 10000, 12), [[16, 32], [8, 16]]),    # two partitions (second one adds)
+                      (mixed_band_matrix(rng, 24000), [[8, 16, 32, 64]])):     # several buckets of one partition
         _, info = check(fa, torch, g, widths, feat, b_dtype, seed=feat)
-        assert info["row_group_buckets"] >= 1, (widths, info)
+        assert info["row_group_buckets"] >= (4 if len(widths[0]) == 4 else 1), (widths, info)
         monkeypatch.setenv("LF_ROW_GROUPS", "0")
         _, info_off = check(fa, torch, g, widths, feat, b_dtype, seed=feat)
         monkeypatch.delenv("LF_ROW_GROUPS")
