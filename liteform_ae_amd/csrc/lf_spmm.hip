@@ -803,33 +803,59 @@ rowgroup_count_kernel(const RowGroupCand* __restrict__ cands, unsigned long long
     }
 }
 
-// goff[g] = exclusive prefix of m[g] (in place is not possible: goff has one more entry);
-// single workgroup, the arrays are a few hundred thousand entries.
+// goff[g] = exclusive prefix of m[g], goff[n_groups] = total, in three small launches:
+// sums of blocks of 1024 groups, their exclusive scan by one workgroup (in place, total
+// appended), then the scan inside every block.
+__device__ __forceinline__ int block_inclusive_scan_1024(int x, int* s_wave) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl = x;
+    for (int d = 1; d < 64; d <<= 1) {
+        const int y = __shfl_up(incl, d);
+        if (lane >= d) incl += y;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) incl += s_wave[w];
+    __syncthreads();
+    return incl;
+}
+
 __global__ void __launch_bounds__(1024)
-rowgroup_scan_kernel(const int32_t* __restrict__ m, long long n_groups, int32_t* __restrict__ goff) {
+rowgroup_blocksum_kernel(const int32_t* __restrict__ m, long long n_groups, int32_t* __restrict__ partial) {
+    __shared__ int s_wave[16];
+    const long long i = (long long)blockIdx.x * 1024 + threadIdx.x;
+    const int incl = block_inclusive_scan_1024(i < n_groups ? m[i] : 0, s_wave);
+    if (threadIdx.x == 1023) partial[blockIdx.x] = incl;
+}
+
+__global__ void __launch_bounds__(1024)
+rowgroup_scanpartial_kernel(int32_t* __restrict__ partial, int n_blocks) {
     __shared__ int s_wave[16];
     __shared__ int s_carry;
     if (threadIdx.x == 0) s_carry = 0;
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (long long base = 0; base < n_groups; base += 1024) {
-        const long long i = base + threadIdx.x;
-        const int x = i < n_groups ? m[i] : 0;
-        int incl = x;
-        for (int d = 1; d < 64; d <<= 1) {
-            const int y = __shfl_up(incl, d);
-            if (lane >= d) incl += y;
-        }
-        if (lane == 63) s_wave[wave] = incl;
+    for (int base = 0; base < n_blocks; base += 1024) {
+        const int i = base + threadIdx.x;
+        const int x = i < n_blocks ? partial[i] : 0;
+        const int incl = block_inclusive_scan_1024(x, s_wave);
+        const int carry = s_carry;
+        if (i < n_blocks) partial[i] = carry + incl - x;
         __syncthreads();
-        int off = s_carry;
-        for (int w = 0; w < wave; ++w) off += s_wave[w];
-        if (i < n_groups) goff[i] = off + incl - x;
-        __syncthreads();
-        if (threadIdx.x == 1023) s_carry = off + incl;
+        if (threadIdx.x == 1023) s_carry = carry + incl;
         __syncthreads();
     }
-    if (threadIdx.x == 0) goff[n_groups] = s_carry;
+    if (threadIdx.x == 0) partial[n_blocks] = s_carry;
+}
+
+__global__ void __launch_bounds__(1024)
+rowgroup_scan_kernel(const int32_t* __restrict__ m, long long n_groups, const int32_t* __restrict__ partial,
+                     int n_blocks, int32_t* __restrict__ goff) {
+    __shared__ int s_wave[16];
+    const long long i = (long long)blockIdx.x * 1024 + threadIdx.x;
+    const int x = i < n_groups ? m[i] : 0;
+    const int incl = block_inclusive_scan_1024(x, s_wave);
+    if (i < n_groups) goff[i] = partial[blockIdx.x] + incl - x;
+    if (blockIdx.x == 0 && threadIdx.x == 0) goff[n_groups] = partial[n_blocks];
 }
 
 __global__ void __launch_bounds__(256)
@@ -1448,7 +1474,12 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
                     LF_TRY(dev_alloc(plan, &ecol, (size_t)entries));
                     LF_TRY(dev_alloc(plan, &eval, (size_t)entries));
                     LF_TRY(dev_alloc(plan, &emask, (size_t)entries));
-                    rowgroup_scan_kernel<<<1, 1024, 0, s>>>(m_arrays[i], mb.n_groups, goff);
+                    const int n_blocks = (int)lf::ceil_div(mb.n_groups, 1024);
+                    int32_t* partial = nullptr;
+                    LF_TRY(dev_alloc(plan, &partial, (size_t)n_blocks + 1));
+                    rowgroup_blocksum_kernel<<<n_blocks, 1024, 0, s>>>(m_arrays[i], mb.n_groups, partial);
+                    rowgroup_scanpartial_kernel<<<1, 1024, 0, s>>>(partial, n_blocks);
+                    rowgroup_scan_kernel<<<n_blocks, 1024, 0, s>>>(m_arrays[i], mb.n_groups, partial, n_blocks, goff);
                     LF_TRY_HIP(hipGetLastError());
                     rowgroup_fill_kernel<<<(int)lf::ceil_div(mb.n_groups, 256), 256, 0, s>>>(
                         b.d_cols, b.d_vals, meta[k], b.num_ell_rows, lf::ilog2(b.width), mb.n_groups, goff, ecol, eval, emask);
