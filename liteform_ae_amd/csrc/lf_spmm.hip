@@ -674,7 +674,10 @@ spmm_finalize_kernel(const HeavyRow* __restrict__ heavy, int n_heavy, LaunchArgs
 // time); a matrix without shared columns never does.  Separate kernel, so that its registers
 // (four accumulators) do not weigh on the main one.
 constexpr int kGroupRows = 4;
-constexpr int kMergedCap = 384;        // merged entries staged per workgroup at most
+#ifndef LF_MERGED_CAP
+#define LF_MERGED_CAP 1024
+#endif
+constexpr int kMergedCap = LF_MERGED_CAP;   // merged entries staged per workgroup at most
 constexpr int kMergedTileGroups = 64;  // row groups per tile at most
 constexpr long long kRowGroupMinRows = 4096;   // smaller buckets are not worth the analysis
 constexpr int kRowGroupSample = 4096;          // the decision looks at about this many groups of a bucket first
@@ -897,63 +900,71 @@ spmm_rowgroup_kernel(const MergedBucket* __restrict__ buckets, int n_buckets, La
         const int tid = threadIdx.x;
         for (int i = tid; i <= n; i += kWG) s_goff[i] = b.goff[g0 + i];
         __syncthreads();
-        const int base = s_goff[0];
-        const int n_entries = s_goff[n] - base;            // <= kMergedCap by the choice of groups_per_tile
-        for (int i = tid; i < n_entries; i += kWG) {
-            s_col[i] = b.ecol[base + i];
-            s_val[i] = b.eval[base + i];
-            s_msk[i] = b.emask[base + i];
-        }
-        __syncthreads();
         const int sw = tid / LPR, sl = tid % LPR;
         const Lane<LPR, 1, VEC> ln(sl, a.feat, a.ldb, a.ldc);
-        for (int gi = sw; gi < n; gi += SW) {
-            const int e0 = s_goff[gi] - base;
-            const int m = s_goff[gi + 1] - s_goff[gi];
-            Acc<1, VEC> acc[kGroupRows];
+        // The tile's groups are staged in rounds of as many whole groups as the buffer holds
+        // (one group always fits: the plan checks the longest group against the capacity).
+        for (int ga = 0; ga < n;) {
+            const int base = s_goff[ga];
+            int gb = ga + 1;
+            while (gb < n && s_goff[gb + 1] - base <= kMergedCap) ++gb;      // uniform
+            const int n_entries = s_goff[gb] - base;
+            for (int i = tid; i < n_entries; i += kWG) {
+                s_col[i] = b.ecol[base + i];
+                s_val[i] = b.eval[base + i];
+                s_msk[i] = b.emask[base + i];
+            }
+            __syncthreads();
+            for (int gi = ga + sw; gi < gb; gi += SW) {
+                const int e0 = s_goff[gi] - base;
+                const int m = s_goff[gi + 1] - s_goff[gi];
+                Acc<1, VEC> acc[kGroupRows];
 #pragma unroll
-            for (int r = 0; r < kGroupRows; ++r) acc[r].clear();
-            for (int j = 0; j < m; j += U) {
-                int c[U];
-                float4 w[U];
-                uint32_t k[U];
+                for (int r = 0; r < kGroupRows; ++r) acc[r].clear();
+                for (int j = 0; j < m; j += U) {
+                    int c[U];
+                    float4 w[U];
+                    uint32_t k[U];
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const bool in = j + u < m;
-                    const int idx = e0 + (in ? j + u : 0);   // past the end: the first column again, nothing added
-                    c[u] = s_col[idx];
-                    w[u] = in ? s_val[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
-                    k[u] = in ? s_msk[idx] : 0u;
-                }
-                float x[U][VEC];
+                    for (int u = 0; u < U; ++u) {
+                        const bool in = j + u < m;
+                        const int idx = e0 + (in ? j + u : 0);   // past the end: the first column again, nothing added
+                        c[u] = s_col[idx];
+                        w[u] = in ? s_val[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+                        k[u] = in ? s_msk[idx] : 0u;
+                    }
+                    float x[U][VEC];
 #pragma unroll
-                for (int u = 0; u < U; ++u)
-                    Dense<BT>::load(a.B, (size_t)(uint32_t)c[u] * (size_t)ln.ldb + ln.f[0], x[u]);
+                    for (int u = 0; u < U; ++u)
+                        Dense<BT>::load(a.B, (size_t)(uint32_t)c[u] * (size_t)ln.ldb + ln.f[0], x[u]);
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const float wr[kGroupRows] = {w[u].x, w[u].y, w[u].z, w[u].w};
+                    for (int u = 0; u < U; ++u) {
+                        const float wr[kGroupRows] = {w[u].x, w[u].y, w[u].z, w[u].w};
 #pragma unroll
-                    for (int r = 0; r < kGroupRows; ++r) {
-                        if constexpr (LPR == 64) {
-                            // one group per wavefront: rows without the column are skipped outright
-                            if (__builtin_amdgcn_readfirstlane(k[u]) & (1u << r)) {
+                        for (int r = 0; r < kGroupRows; ++r) {
+                            if constexpr (LPR == 64) {
+                                // one group per wavefront: rows without the column are skipped outright
+                                if (__builtin_amdgcn_readfirstlane(k[u]) & (1u << r)) {
+#pragma unroll
+                                    for (int i = 0; i < VEC; ++i) acc[r].v[0][i] = fmaf(wr[r], x[u][i], acc[r].v[0][i]);
+                                }
+                            } else {
+                                // several groups per wavefront: the value is 0 where the row lacks the
+                                // column (like a padded slot, this adds 0 * B: only non-finite B differs)
 #pragma unroll
                                 for (int i = 0; i < VEC; ++i) acc[r].v[0][i] = fmaf(wr[r], x[u][i], acc[r].v[0][i]);
                             }
-                        } else {
-                            // several groups per wavefront: the value is 0 where the row lacks the
-                            // column (like a padded slot, this adds 0 * B: only non-finite B differs)
-#pragma unroll
-                            for (int i = 0; i < VEC; ++i) acc[r].v[0][i] = fmaf(wr[r], x[u][i], acc[r].v[0][i]);
                         }
                     }
                 }
-            }
 #pragma unroll
-            for (int r = 0; r < kGroupRows; ++r) {
-                const long long e = (g0 + gi) * kGroupRows + r;
-                if (e < b.n_rows) store_row<LPR, 1, VEC>(a.C, b.rows[e], ln, acc[r], a.accumulate);
+                for (int r = 0; r < kGroupRows; ++r) {
+                    const long long e = (g0 + gi) * kGroupRows + r;
+                    if (e < b.n_rows) store_row<LPR, 1, VEC>(a.C, b.rows[e], ln, acc[r], a.accumulate);
+                }
             }
+            ga = gb;
+            if (ga < n) __syncthreads();                 // the buffer is refilled
         }
         return;
     }
@@ -1484,10 +1495,10 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
                     rowgroup_fill_kernel<<<(int)lf::ceil_div(mb.n_groups, 256), 256, 0, s>>>(
                         b.d_cols, b.d_vals, meta[k], b.num_ell_rows, lf::ilog2(b.width), mb.n_groups, goff, ecol, eval, emask);
                     LF_TRY_HIP(hipGetLastError());
-                    // tile: as many groups as the staging buffer surely holds, but enough tiles to spread
-                    long long per_tile = std::min<long long>(kMergedTileGroups, kMergedCap / (long long)longest);
+                    // tile: one group per sub-wave (the tile is staged in rounds when its entries
+                    // exceed the buffer), fewer when the bucket is small
                     const long long spread = lf::ceil_div(mb.n_groups, (long long)4 * plan->num_cus);
-                    per_tile = std::max<long long>(1, std::min(per_tile, std::max<long long>(sw, spread)));
+                    const long long per_tile = std::max<long long>(1, std::min<long long>(std::min(sw, kMergedTileGroups), spread));
                     mb.groups_per_tile = (int)per_tile;
                     mb.n_tiles = lf::ceil_div(mb.n_groups, per_tile);
                     mb.rows = b.d_rows;
