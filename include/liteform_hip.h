@@ -179,6 +179,11 @@ int lf_hyb_build(const int32_t* d_indptr, const int32_t* d_indices, const float*
  * (format_algos.py:552-578: values float32, rows int32, cols int32 row-major), plus the
  * optional meta array of lf_hyb_build (NULL: derived from rows/vals at create time).
  * The slabs must stay alive and unchanged while the plan exists.
+ * At creation, buckets of 8..64-slot rows whose consecutive rows hold mostly the same columns
+ * (stencils, banded and block-structured matrices) are rewritten inside the plan as groups
+ * of four rows with merged column lists, so that one read of a B row serves up to four
+ * output rows; this costs plan time and memory (about 21 bytes per merged entry) only
+ * where a sample of the bucket shows at least 30 % fewer reads.
  * feat_size must be a multiple of 32 (float32 B) or 64 (bf16 B), at most 1024.
  * ------------------------------------------------------------------------------------ */
 typedef struct lf_bucket_desc {
