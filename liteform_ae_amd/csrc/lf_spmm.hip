@@ -1448,7 +1448,8 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
                 c.stride = sample ? (int)std::max<long long>(1, c.n_groups / kRowGroupSample) : 1;
                 most = std::max<long long>(most, lf::ceil_div(c.n_groups, c.stride));
             }
-            LF_HIP(hipMemsetAsync(d_rg, 0, cand.size() * 24, s));
+            fill_bytes_kernel<<<1, 64, 0, s>>>((uint32_t*)d_rg, (long long)cand.size() * 6, 0u);
+            LF_HIP(hipGetLastError());
             LF_HIP(hipMemcpyAsync(d_cands, h_cands.data(), h_cands.size() * sizeof(RowGroupCand), hipMemcpyHostToDevice, s));
             rowgroup_count_kernel<<<dim3((unsigned)lf::ceil_div(most, 256), (unsigned)which.size()), 256, 0, s>>>(d_cands, d_rg);
             LF_HIP(hipGetLastError());
