@@ -328,6 +328,7 @@ def main():
             "traffic": traffic,
             "launches_per_step": parts * windows,
             "kernel_ms": round(kernel_ms, 4),
+            "kernel_ms_median": round(float(np.median(ev_ms)), 4),
             "kernel_ms_min": round(float(np.min(ev_ms)), 4),
             "kernel_ms_cold": round(float(np.mean(ev_cold_ms)), 4),
             "algorithmic_bytes": algo,
