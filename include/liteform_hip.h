@@ -109,6 +109,19 @@ int lf_coo_degrees(const int32_t* d_coo_row, const int32_t* d_coo_col, int64_t n
 int lf_row_features(const int32_t* d_indptr, int64_t num_rows, void* d_scratch,
                     int64_t* h_out /* [4] */, lf_stream_t stream);
 
+/* The same statistics for callers that cannot allocate or bring device scratch memory along:
+ * code recorded into a HIP graph, tight serving loops, harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference.  The four accumulators live in a 32-byte array that is part
+ * of the library's device image (every GPU the library runs on holds its own copy until the
+ * process ends); the function allocates and frees nothing and does not synchronise: d_out
+ * (device memory, int64 [4], 8-byte aligned) receives {min, max, sum, sum of squares} in stream
+ * order.  num_rows above LF_ROW_FEATURES_STATIC_MAX_ROWS is refused with LF_ERR_UNSUPPORTED.
+ * All calls on one GPU share that GPU's array: calls that overlap there (two streams, two
+ * threads) race and must be serialised by the caller. */
+#define LF_ROW_FEATURES_STATIC_MAX_ROWS 2147483646LL
+int lf_row_features_static(const int32_t* d_indptr, int64_t num_rows, int64_t* d_out /* [4] */,
+                           lf_stream_t stream);
+
 /* ------------------------------------------------------------------------------------
  * Bucket-width search on the host (no GPU work).  Replaces modify_single_row_buckets,
  * get_bucket_config, modify_bucket_widths, move_largest_bucket, move_width_one_bucket and

@@ -53,6 +53,7 @@ SIGNATURES = {
                                   i64p, i64p, vp]),
     "lf_coo_degrees": (C.c_int, [vp, vp, C.c_int64, C.c_int64, C.c_int64, C.c_int32, vp, vp]),
     "lf_row_features": (C.c_int, [vp, C.c_int64, vp, vp, vp]),
+    "lf_row_features_static": (C.c_int, [vp, C.c_int64, vp, vp]),
     "lf_search_bucket_config": (C.c_int, [i64p, i64p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                           i32p, i32p, f64p, i32p]),
     "lf_hyb_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int32, C.c_int32]),

@@ -17,9 +17,16 @@
 
 #include <algorithm>
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 #include "lf_internal.h"
+
+// Accumulators of lf_row_features_static: {min, max, sum, sum of squares}.  One copy of the
+// array lives on every GPU the library runs on, for the life of the process.  Host code never
+// uses the array's name as an address: static_scratch() below asks the runtime where the
+// current device keeps it.
+static __device__ __align__(256) unsigned long long lf_static_scratch[4];
 
 namespace {
 
@@ -765,6 +772,59 @@ int lf_row_features(const int32_t* d_indptr, int64_t num_rows, void* d_scratch, 
     LF_HIP(hipGetLastError());
     LF_HIP(hipMemcpyAsync(h_out, acc, 32, hipMemcpyDeviceToHost, s));
     LF_HIP(hipStreamSynchronize(s));
+    return LF_OK;
+}
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+unsigned long long* g_scratch_ptr[kMaxDevices];     // device address of lf_static_scratch, per device
+
+// Address of the current device's copy of lf_static_scratch, looked up once per device.
+int static_scratch(unsigned long long** out) {
+    int dev = -1;
+    LF_HIP(hipGetDevice(&dev));
+    LF_REQUIRE(dev >= 0 && dev < kMaxDevices, LF_ERR_UNSUPPORTED, "device index %d is out of range", dev);
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        LF_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(lf_static_scratch)));
+        LF_REQUIRE(p != nullptr, LF_ERR_HIP, "hipGetSymbolAddress returned a null address");
+        g_scratch_ptr[dev] = (unsigned long long*)p;
+    }
+    *out = g_scratch_ptr[dev];
+    return LF_OK;
+}
+
+__global__ void copy_features_kernel(const unsigned long long* __restrict__ acc, int64_t* __restrict__ out) {
+    if (threadIdx.x < 4) out[threadIdx.x] = (int64_t)acc[threadIdx.x];
+}
+
+}  // namespace
+
+int lf_row_features_static(const int32_t* d_indptr, int64_t num_rows, int64_t* d_out, lf_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    LF_REQUIRE(d_out, LF_ERR_INVALID, "d_out is null");
+    LF_REQUIRE(num_rows >= 0, LF_ERR_INVALID, "bad num_rows");
+    LF_REQUIRE(num_rows <= LF_ROW_FEATURES_STATIC_MAX_ROWS, LF_ERR_UNSUPPORTED,
+               "lf_row_features_static handles at most %lld rows (got %lld)",
+               (long long)LF_ROW_FEATURES_STATIC_MAX_ROWS, (long long)num_rows);
+    LF_REQUIRE(num_rows == 0 || d_indptr, LF_ERR_INVALID, "indptr is null");
+    LF_REQUIRE((uintptr_t)d_out % 8 == 0, LF_ERR_INVALID, "d_out must be 8-byte aligned");
+    unsigned long long* acc = nullptr;
+    if (int rc = static_scratch(&acc)) return rc;
+    // the array keeps the last call's values: min starts at all ones, the rest at zero
+    // (num_rows == 0: the minimum is cleared too, which gives {0, 0, 0, 0})
+    LF_HIP(fill_u32(acc, 2, num_rows > 0 ? 0xFFFFFFFFu : 0u, s));
+    LF_HIP(fill_u32(acc + 1, 6, 0u, s));
+    if (num_rows > 0) {
+        const int grid = (int)std::min<int64_t>((num_rows + kBlock - 1) / kBlock, 1024);
+        row_features_kernel<<<grid, kBlock, 0, s>>>(d_indptr, num_rows, acc);
+        LF_HIP(hipGetLastError());
+    }
+    copy_features_kernel<<<1, 64, 0, s>>>(acc, d_out);
+    LF_HIP(hipGetLastError());
     return LF_OK;
 }
 
