@@ -991,30 +991,155 @@ csr_spmm_kernel(const int32_t* __restrict__ indptr, const int32_t* __restrict__ 
 // ------------------------------------------------------------------------------------
 // Plan-time kernels.
 
-// meta from rows / vals for slabs that come without one: len = position of the last
-// nonzero value + 1 (at least 1); segment counts from runs of equal row ids.
-__global__ void derive_meta_kernel(const int32_t* __restrict__ rows, const float* __restrict__ vals,
-                                   long long n_rows, int log_w, int32_t* __restrict__ meta) {
-    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n_rows) return;
+// Inclusive scans over a 256-thread workgroup: the largest value at or before a thread, the
+// smallest value at or after it.  s_wave: 4 ints of LDS.
+__device__ __forceinline__ int block_scan_max_fwd(int x, int* s_wave) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int d = 1; d < 64; d <<= 1) {
+        const int y = __shfl_up(x, d);
+        if (lane >= d) x = max(x, y);
+    }
+    if (lane == 63) s_wave[wave] = x;
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) x = max(x, s_wave[w]);
+    __syncthreads();
+    return x;
+}
+
+__device__ __forceinline__ int block_scan_min_bwd(int x, int* s_wave) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int d = 1; d < 64; d <<= 1) {
+        const int y = __shfl_down(x, d);
+        if (lane + d < 64) x = min(x, y);
+    }
+    if (lane == 0) s_wave[wave] = x;
+    __syncthreads();
+    for (int w = wave + 1; w < 4; ++w) x = min(x, s_wave[w]);
+    __syncthreads();
+    return x;
+}
+
+// meta from rows / vals for slabs that come without one (the reference passes rows, cols and
+// values only, format_algos.py:552-578): len = position of the last nonzero value + 1 (at
+// least 1); a run of equal row ids is one segment.  Two passes, so that a long run costs a
+// scan and not a walk per ELL row: the first notes, per block of 256 ELL rows, its first and
+// its last segment head (an ELL row whose predecessor carries another row id); the second
+// finds for every ELL row the head at or before it and, for a head, the next head.
+__global__ void __launch_bounds__(256)
+derive_heads_kernel(const int32_t* __restrict__ rows, long long n_rows, int32_t* __restrict__ blk_first,
+                    int32_t* __restrict__ blk_last) {
+    __shared__ int s_wave[4];
+    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    const bool head = e < n_rows && (e == 0 || rows[e - 1] != rows[e]);
+    const int last = block_scan_max_fwd(head ? (int)e : -1, s_wave);
+    const int first = block_scan_min_bwd(head ? (int)e : 0x7FFFFFFF, s_wave);
+    if (threadIdx.x == 255) blk_last[blockIdx.x] = last;
+    if (threadIdx.x == 0) blk_first[blockIdx.x] = first;
+}
+
+// flags[3] is raised when a segment is longer than the meta word can say.
+__global__ void __launch_bounds__(256)
+derive_meta_kernel(const int32_t* __restrict__ rows, const float* __restrict__ vals, long long n_rows,
+                   int log_w, const int32_t* __restrict__ blk_first, const int32_t* __restrict__ blk_last,
+                   int n_blocks, int32_t* __restrict__ meta, int* __restrict__ flags) {
+    __shared__ int s_wave[4];
+    __shared__ int s_prev, s_next;
+    if (threadIdx.x == 0) {                      // heads outside this block (block 0 starts with one)
+        int b = (int)blockIdx.x - 1;
+        while (b >= 0 && blk_last[b] < 0) --b;
+        s_prev = b >= 0 ? blk_last[b] : 0;
+        b = (int)blockIdx.x + 1;
+        while (b < n_blocks && blk_first[b] == 0x7FFFFFFF) ++b;
+        s_next = b < n_blocks ? blk_first[b] : (int)n_rows;
+    }
+    __syncthreads();
+    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    const bool in = e < n_rows;
+    const bool head = in && (e == 0 || rows[e - 1] != rows[e]);
+    int prev = block_scan_max_fwd(head ? (int)e : -1, s_wave);
+    // the next head strictly after e: the smallest head at or after the thread's successor
+    __shared__ int s_at_or_after[257];
+    s_at_or_after[threadIdx.x] = block_scan_min_bwd(head ? (int)e : 0x7FFFFFFF, s_wave);
+    if (threadIdx.x == 0) s_at_or_after[256] = 0x7FFFFFFF;
+    __syncthreads();
+    int next = s_at_or_after[threadIdx.x + 1];
+    if (!in) return;
+    if (prev < 0) prev = s_prev;
+    if (next == 0x7FFFFFFF) next = min(s_next, (int)n_rows);
     const int w = 1 << log_w;
     const float* rv = vals + (e << log_w);
     int len = 1;
     for (int j = w - 1; j > 0; --j)
         if (rv[j] != 0.f) { len = j + 1; break; }
-    const int r = rows[e];
     uint32_t field, cont = 0;
-    if (e > 0 && rows[e - 1] == r) {
-        long long h = e - 1;
-        while (h > 0 && rows[h - 1] == r) --h;
-        field = (uint32_t)(e - h);
-        cont = 0x80000000u;
+    if (head) {
+        field = (uint32_t)(next - (int)e);
     } else {
-        long long t = e + 1;
-        while (t < n_rows && rows[t] == r) ++t;
-        field = (uint32_t)(t - e);
+        field = (uint32_t)((int)e - prev);
+        cont = 0x80000000u;
+    }
+    if (field >= (1u << (31 - kMetaLenBits))) {
+        flags[3] = 1;
+        field = 1;                                 // keep the word well formed; the plan is refused
     }
     meta[e] = (int32_t)((uint32_t)len | (field << kMetaLenBits) | cont);
+}
+
+// Checks what the SpMM kernels take on trust from a bucket: source rows inside the matrix,
+// column indices inside B, 1..W valid slots per ELL row, and segments (a head that announces
+// n ELL rows followed by continuation rows 1..n-1 with the same row id) that are complete
+// and stay inside the bucket.  flags[0] bad column, [1] bad row, [2] bad meta.
+__global__ void __launch_bounds__(256)
+validate_bucket_kernel(const int32_t* __restrict__ rows, const int32_t* __restrict__ meta,
+                       const int32_t* __restrict__ cols, long long n_rows, int log_w,
+                       long long num_rows, long long num_cols, int* __restrict__ flags) {
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    const long long t0 = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    bool bad_col = false, bad_row = false, bad_meta = false;
+    const long long n_slots = n_rows << log_w;
+    for (long long i = t0 * 4; i < n_slots; i += stride * 4) {
+        if (i + 4 <= n_slots) {
+            const int4 c = *reinterpret_cast<const int4*>(cols + i);
+            bad_col |= (unsigned)c.x >= (unsigned long long)num_cols || (unsigned)c.y >= (unsigned long long)num_cols ||
+                       (unsigned)c.z >= (unsigned long long)num_cols || (unsigned)c.w >= (unsigned long long)num_cols;
+        } else {
+            for (long long k = i; k < n_slots; ++k) bad_col |= (unsigned)cols[k] >= (unsigned long long)num_cols;
+        }
+    }
+    for (long long e = t0; e < n_rows; e += stride) {
+        bad_row |= (unsigned)rows[e] >= (unsigned long long)num_rows;
+        const int m = meta[e];
+        const int len = m & (int)kMetaLenMask;
+        bad_meta |= len < 1 || len > (1 << log_w);
+        const long long field = (long long)(((uint32_t)m & 0x7FFFFFFFu) >> kMetaLenBits);
+        // what the next ELL row must be: a continuation row with index `want`, or a head (0)
+        long long want = 0;
+        if (m >= 0) {
+            bad_meta |= field < 1 || e + field > n_rows;
+            want = field > 1 ? 1 : 0;
+        } else {
+            const long long h = e - field;
+            if (field < 1 || h < 0) {
+                bad_meta = true;
+            } else {
+                const int hm = meta[h];
+                const long long n = (long long)((uint32_t)hm >> kMetaLenBits);
+                bad_meta |= hm < 0 || field >= n || rows[h] != rows[e];
+                want = field + 1 < n ? field + 1 : 0;
+            }
+        }
+        if (e == 0) bad_meta |= m < 0;
+        if (e + 1 < n_rows) {
+            const int nm = meta[e + 1];
+            const long long nf = (long long)(((uint32_t)nm & 0x7FFFFFFFu) >> kMetaLenBits);
+            bad_meta |= want == 0 ? nm < 0 : (nm >= 0 || nf != want);
+        } else {
+            bad_meta |= want != 0;
+        }
+    }
+    if (__ballot(bad_col) != 0 && (threadIdx.x & 63) == 0) flags[0] = 1;
+    if (__ballot(bad_row) != 0 && (threadIdx.x & 63) == 0) flags[1] = 1;
+    if (__ballot(bad_meta) != 0 && (threadIdx.x & 63) == 0) flags[2] = 1;
 }
 
 // Finds the source rows of a bucket that take the cooperative path (more than kCoopSlots
@@ -1154,6 +1279,7 @@ struct lf_spmm_plan {
     std::vector<Launch> launches;
     MergedBucket* d_merged = nullptr;   // row-group buckets, grouped by partition
     std::vector<void*> owned;        // device allocations released by destroy
+    std::vector<void*> temp;         // plan-time scratch, released when lf_spmm_create returns
     Group* d_groups = nullptr;
     HeavyRow* d_heavy = nullptr;
     float* d_partials = nullptr;
@@ -1162,14 +1288,22 @@ struct lf_spmm_plan {
 
 namespace {
 
-template <typename T> int dev_alloc(lf_spmm_plan* p, T** out, size_t count) {
+template <typename T> int dev_alloc(lf_spmm_plan* p, T** out, size_t count, bool temporary = false) {
     *out = nullptr;
     if (count == 0) return LF_OK;
     void* ptr = nullptr;
     LF_HIP(hipMalloc(&ptr, count * sizeof(T)));
-    p->owned.push_back(ptr);
+    (temporary ? p->temp : p->owned).push_back(ptr);
     *out = (T*)ptr;
     return LF_OK;
+}
+
+int free_temporaries(lf_spmm_plan* p) {
+    int rc = LF_OK;
+    for (void* ptr : p->temp)
+        if (hipFree(ptr) != hipSuccess) rc = LF_ERR_HIP;
+    p->temp.clear();
+    return rc;
 }
 
 using KernelFn = void (*)(LaunchArgs);
@@ -1240,7 +1374,7 @@ extern "C" {
 
 int lf_spmm_destroy(lf_spmm_plan* plan) {
     if (!plan) return LF_OK;
-    int rc = LF_OK;
+    int rc = free_temporaries(plan);
     for (void* p : plan->owned)
         if (hipFree(p) != hipSuccess) rc = LF_ERR_HIP;
     delete plan;
@@ -1311,10 +1445,11 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     // the counting pass, the filling pass and the coverage pass each cost one copy back and
     // one synchronisation for the whole plan, not one per bucket.
     std::vector<const int32_t*> meta((size_t)num_buckets, nullptr);
-    const int n_counters = 4 * (num_buckets + 1);
+    const int n_counters = 4 * (num_buckets + 2);
     int* d_counters = nullptr;              // [4k .. 4k+3]: plan_chunks_kernel's counters of bucket k
-    LF_TRY(dev_alloc(plan, &d_counters, (size_t)n_counters));
+    LF_TRY(dev_alloc(plan, &d_counters, (size_t)n_counters, true));
     int* d_zero_count = d_counters + 4 * num_buckets;
+    int* d_flags = d_counters + 4 * (num_buckets + 1);   // validate_bucket_kernel, derive_meta_kernel
     std::vector<int> h_counters((size_t)n_counters, 0);
     std::vector<int> is_multi((size_t)num_buckets, 0);
     struct ChunkCount { int chunks = 0, heavy = 0, partials = 0; };
@@ -1343,16 +1478,38 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         if (b.d_meta) {
             meta[k] = b.d_meta;
         } else {
-            int32_t* m = nullptr;
+            int32_t *m = nullptr, *blk_first = nullptr, *blk_last = nullptr;
+            const int n_blocks = (int)((b.num_ell_rows + 255) / 256);
             LF_TRY(dev_alloc(plan, &m, (size_t)b.num_ell_rows));
-            derive_meta_kernel<<<(int)((b.num_ell_rows + 255) / 256), 256, 0, s>>>(b.d_rows, b.d_vals,
-                                                                                   b.num_ell_rows, log_w, m);
+            LF_TRY(dev_alloc(plan, &blk_first, (size_t)n_blocks, true));
+            LF_TRY(dev_alloc(plan, &blk_last, (size_t)n_blocks, true));
+            derive_heads_kernel<<<n_blocks, 256, 0, s>>>(b.d_rows, b.num_ell_rows, blk_first, blk_last);
+            LF_TRY_HIP(hipGetLastError());
+            derive_meta_kernel<<<n_blocks, 256, 0, s>>>(b.d_rows, b.d_vals, b.num_ell_rows, log_w, blk_first,
+                                                        blk_last, n_blocks, m, d_flags);
             LF_TRY_HIP(hipGetLastError());
             meta[k] = m;
+        }
+        {
+            const long long units = std::max<long long>(b.num_ell_rows, ((long long)b.num_ell_rows << log_w) / 4);
+            const int vgrid = (int)std::min<long long>(lf::ceil_div(units, 256), 4096);
+            validate_bucket_kernel<<<vgrid, 256, 0, s>>>(b.d_rows, meta[k], b.d_cols, b.num_ell_rows, log_w,
+                                                         num_rows, num_cols, d_flags);
+            LF_TRY_HIP(hipGetLastError());
         }
         LF_TRY_HIP(launch_plan_chunks(k, nullptr, nullptr, 0, 0));
     }
     LF_TRY_HIP(read_counters());
+    {
+        // nothing below (and no SpMM launch) may run on slabs that fail these checks: a column
+        // or row index out of range would be an out-of-range gather or store
+        const int* f = &h_counters[4 * (num_buckets + 1)];
+        if (f[0]) return bail(lf::fail(LF_ERR_INVALID, "a bucket holds a column index outside [0, %lld)", (long long)num_cols));
+        if (f[1]) return bail(lf::fail(LF_ERR_INVALID, "a bucket holds a row index outside [0, %lld)", (long long)num_rows));
+        if (f[2]) return bail(lf::fail(LF_ERR_INVALID, "a bucket's meta array is inconsistent (valid slots outside 1..W, "
+                                                        "or a segment that is incomplete or leaves the bucket)"));
+        if (f[3]) return bail(lf::fail(LF_ERR_UNSUPPORTED, "a row is split over more than %d ELL rows", (1 << (31 - kMetaLenBits)) - 1));
+    }
     for (int k = 0; k < num_buckets; ++k) {
         counts[k].chunks = h_counters[4 * k + 0];
         counts[k].heavy = h_counters[4 * k + 1];
@@ -1392,7 +1549,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     if (num_rows > 0) {
         const size_t cov_words = ((size_t)num_rows + 3) / 4;
         uint32_t* cov = nullptr;
-        LF_TRY(dev_alloc(plan, &cov, cov_words));
+        LF_TRY(dev_alloc(plan, &cov, cov_words, true));
         d_cov = (uint8_t*)cov;
         fill_bytes_kernel<<<(int)std::min<size_t>((cov_words + 255) / 256, 4096), 256, 0, s>>>(cov, (long long)cov_words, 0u);
         LF_TRY_HIP(hipGetLastError());
@@ -1458,8 +1615,8 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             return LF_OK;
         };
         if (!cand.empty()) {
-            LF_TRY(dev_alloc(plan, &d_rg, cand.size() * 3));
-            LF_TRY(dev_alloc(plan, &d_cands, cand.size()));
+            LF_TRY(dev_alloc(plan, &d_rg, cand.size() * 3, true));
+            LF_TRY(dev_alloc(plan, &d_cands, cand.size(), true));
             LF_TRY(count_pass(cand, true, nullptr));       // a sample of the groups decides
             std::vector<int> chosen;
             for (size_t i = 0; i < cand.size(); ++i)
@@ -1467,7 +1624,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             if (!chosen.empty()) {
                 std::vector<int32_t*> m_arrays(chosen.size(), nullptr);
                 for (size_t i = 0; i < chosen.size(); ++i)
-                    LF_TRY(dev_alloc(plan, &m_arrays[i], (size_t)lf::ceil_div(h_buckets[chosen[i]].num_ell_rows, kGroupRows)));
+                    LF_TRY(dev_alloc(plan, &m_arrays[i], (size_t)lf::ceil_div(h_buckets[chosen[i]].num_ell_rows, kGroupRows), true));
                 LF_TRY(count_pass(chosen, false, &m_arrays));
                 for (size_t i = 0; i < chosen.size(); ++i) {
                     const int k = chosen[i];
@@ -1488,7 +1645,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
                     LF_TRY(dev_alloc(plan, &emask, (size_t)entries));
                     const int n_blocks = (int)lf::ceil_div(mb.n_groups, 1024);
                     int32_t* partial = nullptr;
-                    LF_TRY(dev_alloc(plan, &partial, (size_t)n_blocks + 1));
+                    LF_TRY(dev_alloc(plan, &partial, (size_t)n_blocks + 1, true));
                     rowgroup_blocksum_kernel<<<n_blocks, 1024, 0, s>>>(m_arrays[i], mb.n_groups, partial);
                     rowgroup_scanpartial_kernel<<<1, 1024, 0, s>>>(partial, n_blocks);
                     rowgroup_scan_kernel<<<n_blocks, 1024, 0, s>>>(m_arrays[i], mb.n_groups, partial, n_blocks, goff);
@@ -1648,6 +1805,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     (void)occ;
     plan->info[7] = (int64_t)merged.size();
     LF_TRY_HIP(hipStreamSynchronize(s));     // the tables are complete: the plan may run on any stream
+    if (free_temporaries(plan) != LF_OK) return bail(lf::fail(LF_ERR_HIP, "hipFree failed on plan-time scratch"));
     *out_plan = plan;
     return LF_OK;
 #undef LF_TRY

@@ -203,3 +203,102 @@ def test_gfx950_search_ignores_column_sets(env):
         assert h2 is None
         assert fa.search_from_statistics(s1, h1, cfgm) == fa.search_from_statistics(s2, None, cfgm) \
             == fa.search_bucket_config(g, parts, cfgm)
+
+
+def _tuple_descs(L, torch, rows_nd, cols_nd, vals_nd, widths, metas=None):
+    """lf_bucket_desc array for reference-style slabs (one partition), with the tensors that
+    keep them alive."""
+    keep = []
+    descs = (L.BucketDesc * len(widths))()
+    for b, w in enumerate(widths):
+        r = dev(torch, rows_nd[b], np.int32)
+        c = dev(torch, np.asarray(cols_nd[b]).reshape(-1), np.int32)
+        v = dev(torch, np.asarray(vals_nd[b]).reshape(-1), np.float32)
+        m = dev(torch, metas[b], np.int32) if metas is not None else None
+        keep += [r, c, v, m]
+        descs[b] = L.BucketDesc(int(w), 0, int(r.numel()), r.data_ptr(), c.data_ptr(), v.data_ptr(),
+                                m.data_ptr() if m is not None else None)
+    return descs, keep
+
+
+def test_bad_slabs_are_refused_at_plan_creation(env):
+    """Caller-supplied slabs (the reference hands rows, cols and values to its kernel unchecked,
+    format_algos.py:552-578) are validated before any kernel gathers or stores through them:
+    only the status code is read, no product runs on the bad data."""
+    lib, L, torch = env
+    rng = np.random.default_rng(77)
+    g = skewed_matrix(rng, 600, 500, mean_deg=5, heavy_rows=1, heavy_len=300, values=False)
+    rows, cols = g.coo_mtx.shape
+    cfg = [[1, 2, 4, 8]]
+    rows_nd, cols_nd, mask_nd = O.build_hyb_format_closed_form(g, cfg)
+    rows_nd, cols_nd, mask_nd = rows_nd[0], cols_nd[0], mask_nd[0]
+
+    def create(r, c, v, metas=None):
+        descs, keep = _tuple_descs(L, torch, r, c, v, cfg[0], metas)
+        plan = C.c_void_p()
+        rc = lib.lf_spmm_create(C.byref(plan), descs, len(cfg[0]), 1, rows, cols, 64, 0, None)
+        msg = L.last_error()
+        if rc == 0:
+            assert lib.lf_spmm_destroy(plan) == 0
+        else:
+            assert not plan.value
+        return rc, msg
+
+    assert create(rows_nd, cols_nd, mask_nd)[0] == 0                       # the good slabs pass
+    for bad_col in (cols, -1, 2**31 - 1):
+        c = [a.copy() for a in cols_nd]
+        c[2][len(c[2]) // 2, 1] = bad_col
+        rc, msg = create(rows_nd, c, mask_nd)
+        assert rc == L.LF_ERR_INVALID and "column index" in msg
+    for bad_row in (rows, -5):
+        r = [a.copy() for a in rows_nd]
+        r[1][0] = bad_row
+        rc, msg = create(r, cols_nd, mask_nd)
+        assert rc == L.LF_ERR_INVALID and "row index" in msg
+    # caller-supplied meta: a length above W, a segment that leaves the bucket, an orphan continuation row
+    def good_meta():
+        out = []
+        for b, w in enumerate(cfg[0]):
+            ln = np.maximum(1, (np.asarray(mask_nd[b]) != 0).sum(1)).astype(np.int64)
+            r = np.asarray(rows_nd[b])
+            m = np.zeros(len(r), dtype=np.int64)
+            i = 0
+            while i < len(r):
+                j = i
+                while j + 1 < len(r) and r[j + 1] == r[i]:
+                    j += 1
+                m[i] = ln[i] | ((j - i + 1) << 11)
+                for t in range(i + 1, j + 1):
+                    m[t] = ln[t] | ((t - i) << 11) | (1 << 31)
+                i = j + 1
+            out.append(m.astype(np.uint32).view(np.int32))
+        return out
+    assert create(rows_nd, cols_nd, mask_nd, good_meta())[0] == 0
+    m = good_meta(); m[0][3] = 2 | (1 << 11)                               # 2 valid slots in a 1-wide row
+    assert create(rows_nd, cols_nd, mask_nd, m)[0] == L.LF_ERR_INVALID
+    m = good_meta(); m[3][-1] = int(m[3][-1] & 0x7FF) | (5 << 11)          # head announcing rows past the end
+    rc, msg = create(rows_nd, cols_nd, mask_nd, m)
+    assert rc == L.LF_ERR_INVALID and "meta" in msg
+    m = good_meta(); m[1][0] = np.int32(-(2**31) + (1 << 11) + 1)          # continuation row with no head
+    assert create(rows_nd, cols_nd, mask_nd, m)[0] == L.LF_ERR_INVALID
+
+
+def test_derived_meta_of_long_segments(env):
+    """Slabs without meta whose widest bucket holds rows split over hundreds of ELL rows (runs
+    of equal row ids crossing several 256-row blocks of the derivation pass)."""
+    lib, L, torch = env
+    from liteform_ae_amd import format_algos as fa
+    rng = np.random.default_rng(78)
+    g = skewed_matrix(rng, 900, 4000, mean_deg=3, heavy_rows=3, heavy_len=2500, values=False)
+    rows, cols = g.coo_mtx.shape
+    cfg = [[1, 2]]
+    hyb = O.build_hyb_format_closed_form(g, cfg)
+    assert max(np.bincount(hyb[0][0][1])) > 600                             # one row id on > 600 ELL rows
+    B = rng.uniform(-1, 1, size=(cols, 32)).astype(np.float32)
+    plan = fa.HybSpMM(hyb, 32, num_rows=rows, num_cols=cols, bucket_widths=cfg)
+    out = plan.run(torch.from_numpy(B).cuda()).cpu().numpy()
+    plan.close()
+    indptr, indices, data = g.adj_tensors("csr")
+    ref = O.spmm_csr_f64(indptr, indices, data, (rows, cols), B)
+    bound = O.spmm_abs_bound(indptr, indices, data, (rows, cols), B)
+    assert (np.abs(out - ref) <= 1e-5 * bound).all()

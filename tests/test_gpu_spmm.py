@@ -203,7 +203,7 @@ def test_stale_output_is_overwritten(fa, torch):
     assert torch.equal(c0, junk)
 
 
-def test_reference_style_driver_flow(fa, torch):
+def test_reference_style_driver_flow(fa, torch, monkeypatch):
     """proc05.spmm.end-to-end.py:153-176 with ones as features and the mask as values."""
     rng = np.random.default_rng(21)
     g = skewed_matrix(rng, 1200, 1200, mean_deg=6, heavy_rows=2, values=False)
@@ -212,9 +212,8 @@ def test_reference_style_driver_flow(fa, torch):
     x = torch.ones((g.num_dst_nodes(), feat))
     y = g.dot(x.numpy())
     hyb = fa.build_hyb_format(g, cfg)
-    import os
-    os.environ["LF_REPEAT"] = "3"
-    os.environ["LF_WARMUP"] = "1"
+    monkeypatch.setenv("LF_REPEAT", "3")
+    monkeypatch.setenv("LF_WARMUP", "1")
     ms = fa.bench_hyb_with_config(g, x, y, feat_size=feat, bucket_widths=cfg, bucketing_format=hyb,
                                   coarsening_factor=2, num_col_parts=parts, use_implicit_unroll=True,
                                   check_correctness=True)
@@ -244,7 +243,7 @@ def test_workloads_scaled(fa, torch):
         check(fa, torch, wl.matrix, cfg, wl.feat_size, wl.b_dtype, seed=wl.seed)
 
 
-def test_partition_chooser_and_driver_table(fa, torch):
+def test_partition_chooser_and_driver_table(fa, torch, monkeypatch):
     from liteform_ae_amd import driver
     rng = np.random.default_rng(41)
     g = skewed_matrix(rng, 3000, 3000, mean_deg=8, heavy_rows=2, values=False)
@@ -252,9 +251,8 @@ def test_partition_chooser_and_driver_table(fa, torch):
     best, timings = fa.choose_num_partitions(g, 64, candidates=(1, 2), return_timings=True)
     assert best in timings and set(timings) == {1, 2}
     assert fa.guess_num_partitions(g, 64) == 1            # B is far smaller than the memory-side cache
-    import os
-    os.environ["LF_REPEAT"] = "2"
-    os.environ["LF_WARMUP"] = "1"
+    monkeypatch.setenv("LF_REPEAT", "2")
+    monkeypatch.setenv("LF_WARMUP", "1")
     df = driver.run_end_to_end([g], feat_sizes=(32, 64), num_parts=2, check_correctness=True)
     assert list(df.columns[:8]) == ["name", "format", "feat_size", "num_parts", "time_select(s)",
                                     "time_num_parts(s)", "time_bucket(s)", "time_exe_our(ms)"]
