@@ -183,6 +183,7 @@ def main():
     ap.add_argument("--windows", type=int, default=0,
                     help="feature windows per step (0 = by measurement together with the partitions)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the matrix (testing only)")
+    ap.add_argument("--b-dtype", default="", choices=["", "f32", "bf16"], help="dtype of B (default: the workload's)")
     ap.add_argument("--cost-model", default="gfx950", choices=["reference", "gfx950"],
                     help="cost function of the bucket-width search (the reference's, or the MI355X one)")
     ap.add_argument("--widths", default="", help="bucket widths instead of the searched ones, "
@@ -211,6 +212,8 @@ def main():
 
     t0 = time.perf_counter()
     wl = make_workload(args.workload, args.scale)
+    if args.b_dtype:
+        wl.b_dtype = args.b_dtype
     feat = args.feat or wl.feat_size
     parts = args.parts or wl.num_parts
     g = wl.matrix

@@ -16,7 +16,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "liblfhip.so")
 
-SOURCES = ["lf_error.cpp", "lf_search.cpp", "lf_format.hip", "lf_spmm.hip", "lf_bsr.hip", "lf_ingest.hip"]
+SOURCES = ["lf_error.cpp", "lf_search.cpp", "lf_format.hip", "lf_spmm.hip", "lf_cells.hip", "lf_bsr.hip", "lf_ingest.hip"]
 
 # -ffp-contract=off: the width search must add and multiply doubles exactly like CPython.
 # packed-fp32-ops is switched off for device code on purpose (scalar fp32 FMAs only).

@@ -1,0 +1,552 @@
+// Cells: shared gathers for structured matrices on gfx950.
+//
+// In a stencil, banded or block-structured matrix the rows that are close together in the
+// underlying grid hold mostly the same columns.  The reference's kernel reads a row of B once
+// per stored entry whatever the structure (playground_pipline/format_algos.py:99-102 under the
+// schedule of 508-533).  Here a bucket of such rows is rewritten at plan time as cells: up to
+// 16 rows that are neighbours in up to three directions (consecutive rows, rows one grid line
+// apart, rows one grid plane apart), with the union of their columns ("merged entries") and,
+// per merged entry, one weight per row of the cell (0 where the row lacks the column).  One
+// 64-lane wavefront owns a cell: it reads each row of B of the union once (16 bytes per lane)
+// and adds weight x row to all 16 accumulator rows at once.  A 4 x 2 x 2 cell of a 27-point
+// stencil reads 96 rows of B for 16 output rows, 6 per row, where row by row it would read 27
+// and four consecutive rows at a time 13.5.
+//
+// The update "16 rows += 16 weights (x) one row of B" is a rank-1 update, and the matrix
+// pipe has an instruction for exactly that: v_mfma_f32_16x16x1_4b_f32 forms four 16 x 16
+// outer products (fp32 in, fp32 accumulate) per issue.  Written with vector FMAs the same cell
+// takes 18 FMAs and ~30 scalar mask tests per merged entry, and rocprofv3 counters showed the
+// kernel bound by instruction issue (one instruction per ~4.7 cycles and SIMD, 0.88 ms for the
+// 100^3 stencil at N = 256, 0.79 ms with the gathers taken out); with four matrix instructions
+// per entry the arithmetic is no longer what binds.  This is not a GEMM formulation: data
+// layout, gathers and accumulation order are the plain path's, only the accumulate instruction
+// differs, and rows that lack a column add 0 * B (as padded slots do).
+//
+// Which rows are neighbours is found from the matrix itself: in a sample of rows, the most
+// frequent differences between two columns of one row are the row distances at which rows
+// share columns (1, 100 and 10000 for a 27-point stencil on a 100^3 grid).  Rows are binned
+// into cells by their coordinates along those strides; the rewrite is kept only when the
+// cells' unions are at most 70 % of the gathers the plain path would issue.
+//
+// A row's terms are added in ascending column order, as in the plain path.
+#include "lf_cells.h"
+
+#include <algorithm>
+#include <cstdlib>
+
+#include "lf_spmm_device.h"
+
+namespace {
+
+constexpr int kCellRows = 16;              // rows of a cell: the row dimension of the outer-product instruction
+constexpr int kCellBatch = 8;              // merged entries are padded to whole batches of this many
+constexpr int kCellTileCells = 4;          // cells a workgroup is on at a time: one per wavefront
+#ifndef LF_CELLS_PER_WAVE
+#define LF_CELLS_PER_WAVE 1
+#endif
+constexpr int kCellsPerWave = LF_CELLS_PER_WAVE;   // cells a wavefront walks one after the other (<= 15)
+constexpr int kCellWidthMax = 64;          // widest bucket that is looked at
+constexpr int kCellSampleRows = 64;        // rows looked at to find the strides
+constexpr int kCellSampleCols = 32;        // ... and how many of each row's columns
+constexpr int kCellMaxPercent = 70;        // merged entries / plain gathers at most, in percent
+constexpr long long kL2BytesPerXcd = 4ll << 20;
+
+// Where a row lies along the strides: cell = ((z / g2) * n1 + y / g1) * n0 + x / g0 with
+// x = (r mod s2) / s1, y = (r mod s3) / s2, z = r / s3 (fewer terms with fewer strides).
+struct CellGeom {
+    int k;                     // strides in use: 1..3
+    int g0, g1, g2;            // rows of a cell along each stride
+    long long s1, s2, s3;
+    long long n0, n1, n2;      // cells along x, y and z
+    int yb;                    // three strides: cell rows along y that are swept through all z before the next ones
+};
+
+__device__ __forceinline__ long long cell_of(const CellGeom& q, long long r) {
+    long long x, y = 0, z = 0;
+    if (q.k == 1) {
+        x = r / q.s1;
+    } else if (q.k == 2) {
+        x = (r % q.s2) / q.s1;
+        y = r / q.s2;
+    } else {
+        x = (r % q.s2) / q.s1;
+        y = (r % q.s3) / q.s2;
+        z = r / q.s3;
+    }
+    const long long xc = x / q.g0, yc = y / q.g1, zc = z / q.g2;
+    if (q.k == 3 && q.yb > 0) return (((yc / q.yb) * q.n2 + zc) * q.yb + yc % q.yb) * q.n0 + xc;
+    return (zc * q.n1 + yc) * q.n0 + xc;
+}
+
+// sample[i] = {source row, valid slots, columns...} of every stride-th ELL row
+__global__ void cell_sample_kernel(const int32_t* __restrict__ rows, const int32_t* __restrict__ cols,
+                                   const int32_t* __restrict__ meta, long long n_rows, int log_w,
+                                   long long stride, int n_samples, int n_cols, int32_t* __restrict__ out) {
+    const int i = blockIdx.x;
+    if (i >= n_samples) return;
+    const long long e = (long long)i * stride;
+    if (e >= n_rows) return;
+    int32_t* o = out + (size_t)i * (n_cols + 2);
+    const int len = meta[e] & (int)kMetaLenMask;
+    if (threadIdx.x == 0) {
+        o[0] = rows[e];
+        o[1] = len;
+    }
+    for (int j = threadIdx.x; j < n_cols; j += blockDim.x) o[2 + j] = j < len ? cols[(e << log_w) + j] : -1;
+}
+
+// perm[cell * G + i] = the i-th ELL row that falls into the cell, in arrival order (the merge
+// pass sorts them); flags[0] is raised when a cell receives more than G rows.
+__global__ void __launch_bounds__(256)
+cell_assign_kernel(const int32_t* __restrict__ rows, long long n_rows, CellGeom q, int G,
+                   int32_t* __restrict__ cnt, int32_t* __restrict__ perm, int* __restrict__ flags) {
+    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n_rows) return;
+    const long long c = cell_of(q, rows[e]);
+    const int pos = atomicAdd(&cnt[c], 1);
+    if (pos < G) perm[c * G + pos] = (int32_t)e;
+    else flags[0] = 1;
+}
+
+// ascending sort inside every group of 16 lanes
+__device__ __forceinline__ unsigned group16_sort_ascending(unsigned v, int lane) {
+    for (int k = 2; k <= 16; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            const unsigned o = __shfl_xor(v, j);
+            const bool up = (lane & k) == 0 || k == 16;
+            const bool lower = (lane & j) == 0;
+            v = (lower == up) ? min(v, o) : max(v, o);
+        }
+    return v;
+}
+
+struct CellMergeArgs {
+    const int32_t* rows;       // the bucket's slab
+    const int32_t* cols;
+    const float* vals;
+    const int32_t* meta;
+    int log_w;
+    long long n_cells;
+    const int32_t* perm;       // [n_cells * 16] ELL rows of each cell in arrival order, -1 = none
+    // counting pass
+    int32_t* m_out;            // [n_cells] merged entries, rounded up to whole batches
+    unsigned long long* stats; // [0] merged entries (not rounded), [1] gathers of the plain path, [2] rounded entries, [3] most rounded entries
+    // writing pass (ecol != nullptr)
+    const int32_t* eoff;
+    int32_t* ecol;
+    float* wq;                 // float4 per (four consecutive entries, row): [entry / 4][16][entry % 4]
+    int32_t* rows_out;         // [n_cells * 16]
+};
+
+// Four cells per 64-thread workgroup, one lane per row of a cell.  The rows' slots are staged
+// in LDS; then the 16 (ascending) column lists of a cell are merged step by step: the smallest
+// head column is the next merged entry, every row that holds it supplies its value and moves
+// on, the others supply 0.  The counting pass only counts the steps; the writing pass stores
+// columns and weights, and pads each cell to whole batches with its last column and zero
+// weights.  No atomics on the output, so the cells do not depend on scheduling.
+__global__ void __launch_bounds__(64)
+cell_merge_kernel(CellMergeArgs a) {
+    constexpr int G = kCellRows;
+    __shared__ int32_t s_c[64 * kCellWidthMax];
+    __shared__ float s_v[64 * kCellWidthMax];
+    const int lane = threadIdx.x, r = lane & 15, g0 = lane & 48;
+    const long long cell = (long long)blockIdx.x * 4 + (lane >> 4);
+    const bool live = cell < a.n_cells;
+    const bool write = a.ecol != nullptr;
+    const int w = 1 << a.log_w;
+
+    unsigned e = 0x7FFFFFFFu;
+    if (live) {
+        const int32_t p = a.perm[cell * G + r];
+        if (p >= 0) e = (unsigned)p;
+    }
+    e = group16_sort_ascending(e, lane);           // ELL rows ascend with the source rows
+    const bool have = e != 0x7FFFFFFFu;
+    if (write && live) a.rows_out[cell * G + r] = have ? a.rows[e] : -1;
+    const int len = have ? (a.meta[e] & (int)kMetaLenMask) : 0;
+    for (int i = 0; i < G; ++i) {                  // row i of each group, 16 slots at a time
+        const long long ei = __shfl(e, g0 + i);
+        const int li = __shfl(len, g0 + i);
+        for (int j = r; j < li; j += 16) {
+            s_c[(g0 + i) * w + j] = a.cols[(ei << a.log_w) + j];
+            if (write) s_v[(g0 + i) * w + j] = a.vals[(ei << a.log_w) + j];
+        }
+    }
+    __syncthreads();
+    int plain = (len + kUnroll - 1) / kUnroll * kUnroll;
+    for (int d = 8; d > 0; d >>= 1) plain += __shfl_xor(plain, d);
+    const int eo = (write && live) ? a.eoff[cell] : 0;
+    const int m8 = (write && live) ? a.eoff[cell + 1] - eo : 0;
+    int pos = 0, cnt = 0, last_col = 0;
+    int head = pos < len ? s_c[lane * w] : 0x7FFFFFFF;
+    for (;;) {
+        int cmin = head;
+        for (int d = 8; d > 0; d >>= 1) cmin = min(cmin, __shfl_xor(cmin, d));
+        const bool any = cmin != 0x7FFFFFFF;       // this group still has columns
+        if (__ballot(any) == 0) break;
+        const bool mine = any && head == cmin;
+        if (write && any) {
+            a.wq[((size_t)((eo + cnt) >> 2) * G + r) * 4 + (cnt & 3)] = mine ? s_v[lane * w + pos] : 0.f;
+            if (r == 0) a.ecol[eo + cnt] = cmin;
+        }
+        if (mine) {
+            ++pos;
+            head = pos < len ? s_c[lane * w + pos] : 0x7FFFFFFF;
+        }
+        if (any) {
+            ++cnt;
+            last_col = cmin;
+        }
+    }
+    if (!live) return;
+    if (!write) {
+        if (r == 0) {
+            const int rounded = (cnt + kCellBatch - 1) / kCellBatch * kCellBatch;
+            a.m_out[cell] = rounded;
+            if (cnt > 0) {
+                atomicAdd(&a.stats[0], (unsigned long long)cnt);
+                atomicAdd(&a.stats[1], (unsigned long long)plain);
+                atomicAdd(&a.stats[2], (unsigned long long)rounded);
+                atomicMax(&a.stats[3], (unsigned long long)rounded);
+            }
+        }
+        return;
+    }
+    for (int i = cnt; i < m8; ++i) {               // padding entries
+        a.wq[((size_t)((eo + i) >> 2) * G + r) * 4 + (i & 3)] = 0.f;
+        if (r == 0) a.ecol[eo + i] = last_col;
+    }
+}
+
+__global__ void fill_i32_kernel(int32_t* __restrict__ p, long long n, int32_t value) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
+        p[i] = value;
+}
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+// read-only plan data addressed through the constant address space: loads at wavefront-uniform
+// addresses then go through the scalar cache and are counted apart from the vector loads
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef const i32x4 __attribute__((address_space(4)))* ConstInt4Ptr;
+typedef const f32x4 __attribute__((address_space(1)))* GlobalFloat4Ptr;
+typedef const i32x4 __attribute__((address_space(1)))* GlobalInt4Ptr;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef const u32x4 __attribute__((address_space(1)))* GlobalU32x4Ptr;
+
+// 16 bytes of a row of B as VEC floats
+template <typename BT> __device__ __forceinline__ void unpack_features(const u32x4& r, float (&f)[Dense<BT>::kVec]);
+template <> __device__ __forceinline__ void unpack_features<float>(const u32x4& r, float (&f)[4]) {
+    f[0] = __uint_as_float(r.x); f[1] = __uint_as_float(r.y); f[2] = __uint_as_float(r.z); f[3] = __uint_as_float(r.w);
+}
+template <> __device__ __forceinline__ void unpack_features<bf16_t>(const u32x4& r, float (&f)[8]) {
+    f[0] = __uint_as_float(r.x << 16); f[1] = __uint_as_float(r.x & 0xFFFF0000u);
+    f[2] = __uint_as_float(r.y << 16); f[3] = __uint_as_float(r.y & 0xFFFF0000u);
+    f[4] = __uint_as_float(r.z << 16); f[5] = __uint_as_float(r.z & 0xFFFF0000u);
+    f[6] = __uint_as_float(r.w << 16); f[7] = __uint_as_float(r.w & 0xFFFF0000u);
+}
+
+// The SpMM kernel: one workgroup per four cells, one wavefront per cell, XCD-aware like the
+// other kernels (workgroup i runs on XCD i % 8 and takes the i / 8-th tile of that XCD's
+// contiguous share of every bucket).  Per merged entry a wavefront gathers one row of B (lane l
+// holds features VEC*l .. VEC*l+VEC-1) and issues VEC matrix instructions: instruction c takes
+// the entry's 16 weights (lane l supplies the weight of row l % 16) and the c-th feature of
+// every lane, and adds the four 16 x 16 outer products to accumulator c.  In accumulator c,
+// register g of lane l belongs to row 4*(l/16) + g%4 and feature VEC*(16*(g/4) + l%16) + c.
+// Entries are walked in half-batches of four: while one is added, the other's loads are in flight.
+template <typename BT>
+__global__ void __launch_bounds__(kWG)
+spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const void* __restrict__ B,
+                 float* __restrict__ C, int feat, int ldb, int ldc, int accumulate) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int G = kCellRows;
+    constexpr int H = 4;
+    const int xcd = blockIdx.x % kXcds;
+    long long v = blockIdx.x / kXcds;
+    for (int bi = 0; bi < n_buckets; ++bi) {
+        const LfCellBucket& b = buckets[bi];
+        const long long lo = b.n_tiles * xcd / kXcds;
+        const long long hi = b.n_tiles * (xcd + 1) / kXcds;
+        if (v >= hi - lo) { v -= hi - lo; continue; }
+        // everything that steers the walk is the same for all lanes of a wavefront
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int lane = threadIdx.x & 63;
+        // A wavefront walks kCellsPerWave cells one after the other (at each step the four
+        // wavefronts of the workgroup are on four neighbouring cells).  One cell per wavefront
+        // measured fastest (100^3 stencil, N = 256: 0.76 / 0.80 / 1.01 ms for 1 / 2 / 4 cells).
+        const long long first = (lo + v) * (kCellTileCells * kCellsPerWave);
+        int my_off = 0;
+        if (first + lane <= b.n_cells) my_off = b.eoff[first + lane];
+        else my_off = b.eoff[b.n_cells];
+        const Lane<64, 1, VEC> ln(lane, feat, ldb, ldc);
+        for (int step = 0; step < kCellsPerWave; ++step) {
+        const int slot = step * kCellTileCells + wave;
+        const long long cell = first + slot;
+        if (cell >= b.n_cells) break;
+        const int e0 = __builtin_amdgcn_readlane(my_off, slot);
+        const int m = __builtin_amdgcn_readlane(my_off, slot + 1) - e0;           // a multiple of kCellBatch
+        if (m == 0) continue;
+        const int32_t* __restrict__ ecol = b.ecol + e0;
+        // (pointers read out of the bucket record are generic to the compiler; saying that they
+        // are global memory keeps their loads off the LDS counter)
+        const GlobalFloat4Ptr wq = reinterpret_cast<GlobalFloat4Ptr>(reinterpret_cast<uintptr_t>(b.wq)) +
+                                   ((size_t)e0 / 4 * G + (lane & 15));
+        floatx16 acc[VEC];
+#pragma unroll
+        for (int c = 0; c < VEC; ++c)
+#pragma unroll
+            for (int g = 0; g < 16; ++g) acc[c][g] = 0.f;
+        // A gather is "row base (the same for all lanes, scalar registers) + 16 * lane": no
+        // per-load address registers, and the 16 bytes stay packed until they are used.
+        const char* b_bytes = reinterpret_cast<const char*>(B);
+        const size_t row_bytes = (size_t)ldb * sizeof(BT);
+        const uint32_t lane_off = (uint32_t)lane * 16u;
+        auto issue = [&](int j, f32x4& w, u32x4 (&x)[H]) {
+            // (no branch around the loads: the compiler counts outstanding loads per path)
+            const int jj = j < m ? j : m - H;                 // past the end: the last half-batch again, unused
+            // the columns come through the scalar cache (wavefront-uniform addresses): a vector
+            // load here would have to be waited for in order, behind the gathers still in flight
+            const i32x4 cols4 = *reinterpret_cast<ConstInt4Ptr>(reinterpret_cast<uintptr_t>(ecol + jj));
+            const int c[H] = {cols4.x, cols4.y, cols4.z, cols4.w};
+            w = wq[(size_t)(jj >> 2) * G];
+#pragma unroll
+            for (int u = 0; u < H; ++u) {
+                const char* row = b_bytes + (size_t)(uint32_t)c[u] * row_bytes;
+                x[u] = *reinterpret_cast<GlobalU32x4Ptr>(reinterpret_cast<uintptr_t>(row + lane_off));
+            }
+        };
+        auto add_rows = [&](const f32x4& w, const u32x4 (&x)[H]) {
+            const float wu[H] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int u = 0; u < H; ++u) {
+                float f[VEC];
+                unpack_features<BT>(x[u], f);
+#pragma unroll
+                for (int c = 0; c < VEC; ++c)
+                    acc[c] = __builtin_amdgcn_mfma_f32_16x16x1f32(wu[u], f[c], acc[c], 0, 0, 0);
+            }
+        };
+        f32x4 wa, wb;
+        u32x4 xa[H], xb[H];
+        // The scheduling fences keep each group of loads ahead of the arithmetic of the other
+        // half-batch; left alone, the compiler sinks the loads to just before their first use
+        // and every half-batch waits out the full memory latency.
+        issue(0, wa, xa);
+        for (int j = 0; j < m; j += 2 * H) {
+            issue(j + H, wb, xb);
+            __builtin_amdgcn_sched_barrier(0);
+            add_rows(wa, xa);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(j + 2 * H, wa, xa);
+            __builtin_amdgcn_sched_barrier(0);
+            add_rows(wb, xb);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // rows of this lane's registers: 4*(lane/16) .. +3
+        const i32x4 my_rows = *reinterpret_cast<GlobalInt4Ptr>(reinterpret_cast<uintptr_t>(b.rows + cell * G + 4 * (lane >> 4)));
+        const int row_of[4] = {my_rows.x, my_rows.y, my_rows.z, my_rows.w};
+#pragma unroll
+        for (int g = 0; g < 16; ++g) {
+            const int row = row_of[g & 3];
+            if (row < 0) continue;
+            float* dst = C + (size_t)row * ldc + VEC * (16 * (g >> 2) + (lane & 15));
+#pragma unroll
+            for (int i = 0; i < VEC; i += 4) {
+                float4 o = make_float4(acc[i][g], acc[i + 1][g], acc[i + 2][g], acc[i + 3][g]);
+                if (accumulate) {
+                    const float4 old = *reinterpret_cast<const float4*>(dst + i);
+                    o.x += old.x; o.y += old.y; o.z += old.z; o.w += old.w;
+                }
+                *reinterpret_cast<float4*>(dst + i) = o;
+            }
+        }
+        }
+        return;
+    }
+}
+
+// Strides and cell shape from a sample of rows.  Returns false when nothing stands out.
+bool detect_geometry(const std::vector<int32_t>& sample, int n_samples, int n_cols, int cell_rows,
+                     int64_t num_rows, long long bucket_rows, long long row_bytes, CellGeom* out, long long* n_cells) {
+    std::vector<long long> diffs;
+    int rows_seen = 0;
+    for (int i = 0; i < n_samples; ++i) {
+        const int32_t* o = sample.data() + (size_t)i * (n_cols + 2);
+        const int len = std::min<int>(o[1], n_cols);
+        if (len < 2) continue;
+        ++rows_seen;
+        for (int x = 0; x < len; ++x)
+            for (int y = x + 1; y < len; ++y) {
+                const long long d = std::llabs((long long)o[2 + y] - (long long)o[2 + x]);
+                if (d > 0) diffs.push_back(d);
+            }
+    }
+    if (rows_seen == 0 || diffs.empty()) return false;
+    std::sort(diffs.begin(), diffs.end());
+    std::vector<std::pair<long long, int>> runs;      // (difference, how often)
+    for (size_t i = 0; i < diffs.size();) {
+        size_t j = i;
+        while (j < diffs.size() && diffs[j] == diffs[i]) ++j;
+        runs.emplace_back(diffs[i], (int)(j - i));
+        i = j;
+    }
+    int top = 0;
+    for (auto& r : runs) top = std::max(top, r.second);
+    if (top < rows_seen) return false;               // no difference that most rows show
+    std::vector<long long> cand;                     // ascending
+    for (auto& r : runs)
+        if ((long long)r.second * 4 >= (long long)top * 3) cand.push_back(r.first);
+    if (cand.empty() || cand[0] != 1) return false;  // rows that share columns must include neighbours
+    auto first_at_least = [&](long long lo) -> long long {
+        for (long long c : cand)
+            if (c >= lo) return c;
+        return 0;
+    };
+    CellGeom q{};
+    q.s1 = 1;
+    const int g3[3] = {4, 2, cell_rows / 8};         // three strides: 4 x 2 x 2
+    const int g2[2] = {4, cell_rows / 4};            // two strides: 4 x 4
+    const long long s2_3 = first_at_least((long long)g3[0]);
+    const long long s3_3 = s2_3 ? first_at_least(s2_3 * g3[1]) : 0;
+    const long long s2_2 = first_at_least((long long)g2[0]);
+    if (s2_3 && s3_3) {
+        q.k = 3; q.g0 = g3[0]; q.g1 = g3[1]; q.g2 = g3[2]; q.s2 = s2_3; q.s3 = s3_3;
+        q.n0 = lf::ceil_div(q.s2, q.g0);
+        q.n1 = lf::ceil_div(lf::ceil_div(q.s3, q.s2), q.g1);
+        q.n2 = lf::ceil_div(lf::ceil_div(num_rows, q.s3), q.g2);
+        // Order of the cells: in plain (z, y, x) order the planes of B that two z-layers of
+        // cells share come round again a whole layer later, long after they left the L2.  So
+        // yb cell rows along y are swept through all z before the next ones, with yb the
+        // largest count whose rows of B for one z-step - (yb * g1 + 2) grid lines of s2 / s1
+        // rows in g2 + 2 planes - fit one XCD's 4 MB L2 (100^3 stencil, 1 KB rows: 4; measured
+        // L2 misses 28.4M / 40.8M / 30.7M / 22.2M / 24.4M for plain order / 1 / 2 / 4 / 8).
+        const long long line_bytes = (q.s2 / q.s1) * (long long)(q.g2 + 2) * row_bytes;
+        const long long lines = line_bytes > 0 ? kL2BytesPerXcd / line_bytes : 0;
+        long long yb = (lines - 2) / q.g1;
+        const char* env_yb = getenv("LF_CELL_YB");
+        if (env_yb) yb = atoi(env_yb);
+        q.yb = (yb >= 2 && yb < q.n1) ? (int)yb : 0;
+        *n_cells = (q.yb > 0 ? lf::ceil_div(q.n1, q.yb) * q.yb : q.n1) * q.n0 * q.n2;
+    } else if (s2_2) {
+        q.k = 2; q.g0 = g2[0]; q.g1 = g2[1]; q.g2 = 1; q.s2 = s2_2; q.s3 = 1;
+        q.n0 = lf::ceil_div(q.s2, q.g0);
+        q.n1 = lf::ceil_div(lf::ceil_div(num_rows, q.s2), q.g1);
+        *n_cells = q.n0 * q.n1;
+    } else {
+        q.k = 1; q.g0 = cell_rows; q.g1 = q.g2 = 1; q.s2 = q.s3 = 1;
+        q.n0 = lf::ceil_div(num_rows, q.g0);
+        q.n1 = 1;
+        *n_cells = q.n0;
+    }
+    // cells that stay mostly empty (a bucket that holds few of the matrix's rows) are not worth it
+    if (*n_cells > 2 * lf::ceil_div(bucket_rows, cell_rows) + 4096 || *n_cells * cell_rows >= (1ll << 31)) return false;
+    *out = q;
+    return true;
+}
+
+template <typename T> int cell_alloc(std::vector<void*>* keep, T** out, size_t count) {
+    *out = nullptr;
+    void* p = nullptr;
+    LF_HIP(hipMalloc(&p, std::max<size_t>(count, 1) * sizeof(T)));
+    keep->push_back(p);
+    *out = (T*)p;
+    return LF_OK;
+}
+
+}  // namespace
+
+namespace lf {
+
+int cells_build(const lf_bucket_desc& b, const int32_t* d_meta, int64_t num_rows, int64_t row_bytes, hipStream_t s,
+                std::vector<void*>* owned, std::vector<void*>* temp, LfCellBucket* out, bool* accepted) {
+    *accepted = false;
+    constexpr int G = kCellRows;
+    if (b.num_ell_rows < 1 || b.width > kCellWidthMax) return LF_OK;
+    const int log_w = lf::ilog2(b.width);
+    const long long R = b.num_ell_rows;
+
+    // ---- strides from a sample of rows
+    const int n_samples = (int)std::min<long long>(kCellSampleRows, R);
+    const int n_cols = std::min<int>(kCellSampleCols, b.width);
+    int32_t* d_sample = nullptr;
+    if (int rc = cell_alloc(temp, &d_sample, (size_t)n_samples * (n_cols + 2))) return rc;
+    cell_sample_kernel<<<n_samples, 64, 0, s>>>(b.d_rows, b.d_cols, d_meta, R, log_w, R / n_samples, n_samples, n_cols, d_sample);
+    LF_HIP(hipGetLastError());
+    std::vector<int32_t> h_sample((size_t)n_samples * (n_cols + 2));
+    LF_HIP(hipMemcpyAsync(h_sample.data(), d_sample, h_sample.size() * 4, hipMemcpyDeviceToHost, s));
+    LF_HIP(hipStreamSynchronize(s));
+    CellGeom geom{};
+    long long n_cells = 0;
+    if (!detect_geometry(h_sample, n_samples, n_cols, G, num_rows, R, row_bytes, &geom, &n_cells)) return LF_OK;
+
+    // ---- rows into cells, then count what the merged cells would hold
+    int32_t *d_cnt = nullptr, *d_perm = nullptr, *d_m = nullptr, *d_partial = nullptr;
+    unsigned long long* d_stats = nullptr;      // four counters, then (at [6]) the overflow flag
+    if (int rc = cell_alloc(temp, &d_cnt, (size_t)n_cells)) return rc;
+    if (int rc = cell_alloc(temp, &d_perm, (size_t)n_cells * G)) return rc;
+    if (int rc = cell_alloc(temp, &d_m, (size_t)n_cells)) return rc;
+    if (int rc = cell_alloc(temp, &d_partial, (size_t)lf::ceil_div(n_cells, 1024) + 1)) return rc;
+    if (int rc = cell_alloc(temp, &d_stats, 8)) return rc;
+    const int fgrid = (int)std::min<long long>(lf::ceil_div(n_cells * G, 256), 4096);
+    fill_i32_kernel<<<fgrid, 256, 0, s>>>(d_cnt, n_cells, 0);
+    fill_i32_kernel<<<fgrid, 256, 0, s>>>(d_perm, n_cells * G, -1);
+    fill_i32_kernel<<<1, 64, 0, s>>>((int32_t*)d_stats, 16, 0);
+    LF_HIP(hipGetLastError());
+    int* d_flags = (int*)(d_stats + 6);
+    cell_assign_kernel<<<(int)lf::ceil_div(R, 256), 256, 0, s>>>(b.d_rows, R, geom, G, d_cnt, d_perm, d_flags);
+    LF_HIP(hipGetLastError());
+    CellMergeArgs ma{};
+    ma.rows = b.d_rows;
+    ma.cols = b.d_cols;
+    ma.vals = b.d_vals;
+    ma.meta = d_meta;
+    ma.log_w = log_w;
+    ma.n_cells = n_cells;
+    ma.perm = d_perm;
+    ma.m_out = d_m;
+    ma.stats = d_stats;
+    cell_merge_kernel<<<(unsigned)lf::ceil_div(n_cells, 4), 64, 0, s>>>(ma);
+    LF_HIP(hipGetLastError());
+    unsigned long long h_stats[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    LF_HIP(hipMemcpyAsync(h_stats, d_stats, sizeof(h_stats), hipMemcpyDeviceToHost, s));
+    LF_HIP(hipStreamSynchronize(s));
+    const unsigned long long entries = h_stats[0], plain = h_stats[1], rounded = h_stats[2];
+    const int overflow = (int)(h_stats[6] & 0xFFFFFFFFull);
+    if (overflow || entries == 0 || rounded >= (1ull << 31) || entries * 100 > plain * kCellMaxPercent ||
+        h_stats[3] > (unsigned long long)kCellEntriesCap)
+        return LF_OK;
+
+    // ---- offsets and the cells themselves
+    int32_t *d_eoff = nullptr, *d_ecol = nullptr, *d_rows_out = nullptr;
+    float4* d_wq = nullptr;
+    if (int rc = cell_alloc(owned, &d_eoff, (size_t)n_cells + 1)) return rc;
+    if (int rc = cell_alloc(owned, &d_ecol, (size_t)rounded)) return rc;
+    if (int rc = cell_alloc(owned, &d_wq, (size_t)rounded / 4 * G)) return rc;
+    if (int rc = cell_alloc(owned, &d_rows_out, (size_t)n_cells * G)) return rc;
+    LF_HIP(exclusive_scan_i32(d_m, n_cells, d_partial, d_eoff, s));
+    ma.eoff = d_eoff;
+    ma.ecol = d_ecol;
+    ma.wq = reinterpret_cast<float*>(d_wq);
+    ma.rows_out = d_rows_out;
+    cell_merge_kernel<<<(unsigned)lf::ceil_div(n_cells, 4), 64, 0, s>>>(ma);
+    LF_HIP(hipGetLastError());
+    out->n_cells = n_cells;
+    out->n_tiles = lf::ceil_div(n_cells, kCellTileCells * kCellsPerWave);
+    out->eoff = d_eoff;
+    out->ecol = d_ecol;
+    out->wq = d_wq;
+    out->rows = d_rows_out;
+    *accepted = true;
+    return LF_OK;
+}
+
+int cells_launch(const LfCellBucket* d_buckets, int n_buckets, int grid, int b_dtype, const void* B, float* C,
+                 int feat, int ldb, int ldc, int accumulate, hipStream_t s) {
+    if (n_buckets <= 0 || grid <= 0) return LF_OK;
+    LF_REQUIRE(b_dtype == LF_DTYPE_F32, LF_ERR_UNSUPPORTED, "cells are built for fp32 operands only");
+    spmm_cell_kernel<float><<<grid, kWG, 0, s>>>(d_buckets, n_buckets, B, C, feat, ldb, ldc, accumulate);
+    LF_HIP(hipGetLastError());
+    return LF_OK;
+}
+
+}  // namespace lf

@@ -32,176 +32,11 @@
 #include <cstring>
 #include <vector>
 
+#include "lf_cells.h"
 #include "lf_internal.h"
+#include "lf_spmm_device.h"
 
 namespace {
-
-constexpr int kWG = 256;            // threads per workgroup (4 wavefronts)
-#ifndef LF_TILE_SLOTS_PER_SUBWAVE
-#define LF_TILE_SLOTS_PER_SUBWAVE 64
-#endif
-#ifndef LF_UNROLL
-#define LF_UNROLL 8
-#endif
-#ifndef LF_TILE_MIN
-#define LF_TILE_MIN 512
-#endif
-// (col, val) pairs staged in LDS per tile: a fixed amount of work per sub-wave, so narrow
-// feature sizes (many sub-waves per workgroup) get larger tiles.  N = 128 -> 512 slots.
-constexpr int tile_slots(int lpr) {
-    const int n = LF_TILE_SLOTS_PER_SUBWAVE * (kWG / lpr);
-    return n < LF_TILE_MIN ? LF_TILE_MIN : n;
-}
-constexpr int kTileRows = 512;      // ELL rows per tile at most (<= tile_slots)
-#ifndef LF_COOP_SLOTS
-#define LF_COOP_SLOTS 256
-#endif
-#ifndef LF_CHUNK_SLOTS
-#define LF_CHUNK_SLOTS 2048
-#endif
-constexpr int kCoopSlots = LF_COOP_SLOTS;    // a source row with more slab slots is reduced by a whole workgroup
-constexpr int kChunkSlots = LF_CHUNK_SLOTS;  // ... in chunks of this many slots (a whole number of ELL rows)
-constexpr int kXcds = 8;
-constexpr int kPartBytesMax = 16384;   // LDS for per-ELL-row sums of a balanced segment tile at most
-constexpr int kUnroll = LF_UNROLL;  // B-row gathers in flight per sub-wave
-constexpr uint32_t kMetaLenMask = 0x7FFu;
-constexpr int kMetaLenBits = 11;
-
-enum GroupType : int { kEll = 0, kSeg = 1, kZero = 2, kChunk = 3, kEllSeg = 4 };
-
-struct Chunk {
-    long long slot_begin;   // first slot, relative to the bucket's slab
-    int n_slots;
-    int partial;            // index of the partial row this chunk produces; < 0: the chunk is the
-                            // whole source row and goes straight to C
-    int row;                // source row
-    int pad_;
-};
-
-struct HeavyRow {
-    int row;
-    int partial_begin;
-    int n_partials;
-    int pad_;
-};
-
-struct Group {
-    int type;
-    int log_w;
-    int rows_per_tile;
-    int balanced;                 // kEllSeg: per-ELL-row sums through LDS (needs rows_per_tile * N floats)
-    long long n_items;            // ELL rows / rows to clear / chunks
-    long long n_tiles;
-    const int32_t* rows;          // kEll, kSeg: source rows; kZero: rows to clear
-    const int32_t* meta;
-    const int32_t* cols;
-    const float* vals;
-    const Chunk* chunks;          // kChunk
-};
-
-struct LaunchArgs {
-    const Group* groups;
-    int n_groups;
-    int accumulate;               // 0: C = result, 1: C += result
-    int feat;                     // N: features computed by the launch
-    int ldb, ldc;                 // row strides of B and C in elements (N, or more for a feature window)
-    int pad_;
-    const void* B;
-    float* C;
-    float* partials;
-};
-
-// ------------------------------------------------------------------------------------
-// Dense-operand access: VEC features per lane as one 16-byte load.
-template <typename BT> struct Dense;
-
-template <> struct Dense<float> {
-    static constexpr int kVec = 4;
-    __device__ static __forceinline__ void load(const void* B, size_t elem, float (&x)[4]) {
-        const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(B) + elem);
-        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
-    }
-};
-
-struct bf16_t { uint16_t bits; };
-
-template <> struct Dense<bf16_t> {
-    static constexpr int kVec = 8;
-    __device__ static __forceinline__ void load(const void* B, size_t elem, float (&x)[8]) {
-        const uint4 v = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(B) + elem);
-        x[0] = __uint_as_float(v.x << 16); x[1] = __uint_as_float(v.x & 0xFFFF0000u);
-        x[2] = __uint_as_float(v.y << 16); x[3] = __uint_as_float(v.y & 0xFFFF0000u);
-        x[4] = __uint_as_float(v.z << 16); x[5] = __uint_as_float(v.z & 0xFFFF0000u);
-        x[6] = __uint_as_float(v.w << 16); x[7] = __uint_as_float(v.w & 0xFFFF0000u);
-    }
-};
-
-// Accumulator of one sub-wave lane: CH chunks of VEC features.
-template <int CH, int VEC> struct Acc {
-    float v[CH][VEC];
-    __device__ __forceinline__ void clear() {
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) v[c][i] = 0.f;
-    }
-};
-
-// Position of a lane inside the feature dimension.
-template <int LPR, int CH, int VEC> struct Lane {
-    int sl;                 // lane inside the sub-wave
-    int feat;               // N: features this launch computes
-    int ldb, ldc;           // elements between consecutive rows of B and of C (>= N)
-    int f[CH];              // first feature of each chunk (clamped to 0 when outside N)
-    bool on[CH];
-    __device__ __forceinline__ Lane(int sl_, int feat_, int ldb_, int ldc_)
-        : sl(sl_), feat(feat_), ldb(ldb_), ldc(ldc_) {
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int f0 = (c * LPR + sl_) * VEC;
-            on[c] = f0 < feat_;
-            f[c] = on[c] ? f0 : 0;
-        }
-    }
-};
-
-template <int U, int LPR, int CH, typename BT>
-__device__ __forceinline__ void gather_fma(const void* B, const Lane<LPR, CH, Dense<BT>::kVec>& ln,
-                                           const int (&col)[U], const float (&val)[U],
-                                           Acc<CH, Dense<BT>::kVec>& acc) {
-    constexpr int VEC = Dense<BT>::kVec;
-    float x[U][CH][VEC];
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-            Dense<BT>::load(B, (size_t)(uint32_t)col[u] * (size_t)ln.ldb + ln.f[c], x[u][c]);
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) acc.v[c][i] = fmaf(val[u], x[u][c][i], acc.v[c][i]);
-}
-
-template <int LPR, int CH, int VEC>
-__device__ __forceinline__ void store_row(float* C, int row, const Lane<LPR, CH, VEC>& ln,
-                                          const Acc<CH, VEC>& acc, int accumulate) {
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        if (!ln.on[c]) continue;
-        float* dst = C + (size_t)row * ln.ldc + ln.f[c];
-#pragma unroll
-        for (int i = 0; i < VEC; i += 4) {
-            float4 o = make_float4(acc.v[c][i], acc.v[c][i + 1], acc.v[c][i + 2], acc.v[c][i + 3]);
-            if (accumulate) {
-                const float4 old = *reinterpret_cast<const float4*>(dst + i);
-                o.x += old.x; o.y += old.y; o.z += old.z; o.w += old.w;
-            }
-            *reinterpret_cast<float4*>(dst + i) = o;
-        }
-    }
-}
 
 // Sum of `total` consecutive slab slots starting at `base`, streamed by one sub-wave: each
 // lane loads one (col, val), the sub-wave then walks them by shuffle.  Slots past `total`
@@ -806,61 +641,6 @@ rowgroup_count_kernel(const RowGroupCand* __restrict__ cands, unsigned long long
     }
 }
 
-// goff[g] = exclusive prefix of m[g], goff[n_groups] = total, in three small launches:
-// sums of blocks of 1024 groups, their exclusive scan by one workgroup (in place, total
-// appended), then the scan inside every block.
-__device__ __forceinline__ int block_inclusive_scan_1024(int x, int* s_wave) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int incl = x;
-    for (int d = 1; d < 64; d <<= 1) {
-        const int y = __shfl_up(incl, d);
-        if (lane >= d) incl += y;
-    }
-    if (lane == 63) s_wave[wave] = incl;
-    __syncthreads();
-    for (int w = 0; w < wave; ++w) incl += s_wave[w];
-    __syncthreads();
-    return incl;
-}
-
-__global__ void __launch_bounds__(1024)
-rowgroup_blocksum_kernel(const int32_t* __restrict__ m, long long n_groups, int32_t* __restrict__ partial) {
-    __shared__ int s_wave[16];
-    const long long i = (long long)blockIdx.x * 1024 + threadIdx.x;
-    const int incl = block_inclusive_scan_1024(i < n_groups ? m[i] : 0, s_wave);
-    if (threadIdx.x == 1023) partial[blockIdx.x] = incl;
-}
-
-__global__ void __launch_bounds__(1024)
-rowgroup_scanpartial_kernel(int32_t* __restrict__ partial, int n_blocks) {
-    __shared__ int s_wave[16];
-    __shared__ int s_carry;
-    if (threadIdx.x == 0) s_carry = 0;
-    __syncthreads();
-    for (int base = 0; base < n_blocks; base += 1024) {
-        const int i = base + threadIdx.x;
-        const int x = i < n_blocks ? partial[i] : 0;
-        const int incl = block_inclusive_scan_1024(x, s_wave);
-        const int carry = s_carry;
-        if (i < n_blocks) partial[i] = carry + incl - x;
-        __syncthreads();
-        if (threadIdx.x == 1023) s_carry = carry + incl;
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) partial[n_blocks] = s_carry;
-}
-
-__global__ void __launch_bounds__(1024)
-rowgroup_scan_kernel(const int32_t* __restrict__ m, long long n_groups, const int32_t* __restrict__ partial,
-                     int n_blocks, int32_t* __restrict__ goff) {
-    __shared__ int s_wave[16];
-    const long long i = (long long)blockIdx.x * 1024 + threadIdx.x;
-    const int x = i < n_groups ? m[i] : 0;
-    const int incl = block_inclusive_scan_1024(x, s_wave);
-    if (i < n_groups) goff[i] = partial[blockIdx.x] + incl - x;
-    if (blockIdx.x == 0 && threadIdx.x == 0) goff[n_groups] = partial[n_blocks];
-}
-
 __global__ void __launch_bounds__(256)
 rowgroup_fill_kernel(const int32_t* __restrict__ cols, const float* __restrict__ vals,
                      const int32_t* __restrict__ meta, long long n_rows, int log_w, long long n_groups,
@@ -1273,11 +1053,13 @@ struct lf_spmm_plan {
         int group_begin = 0, n_groups = 0, grid = 0;
         int dyn_lds = 0;             // bytes of dynamic LDS (balanced segment tiles)
         int merged_begin = 0, n_merged = 0, merged_grid = 0;   // row-group buckets of this partition
+        int cell_begin = 0, n_cell_buckets = 0, cell_grid = 0; // buckets rewritten as cells
         long long tiles = 0;
         int heavy_begin = 0, n_heavy = 0;
     };
     std::vector<Launch> launches;
     MergedBucket* d_merged = nullptr;   // row-group buckets, grouped by partition
+    LfCellBucket* d_cells = nullptr;    // buckets rewritten as cells, grouped by partition
     std::vector<void*> owned;        // device allocations released by destroy
     std::vector<void*> temp;         // plan-time scratch, released when lf_spmm_create returns
     Group* d_groups = nullptr;
@@ -1580,6 +1362,8 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     // ---- row groups: buckets whose consecutive rows share most of their columns
     std::vector<MergedBucket> merged;                      // in bucket (hence partition) order
     std::vector<int> merged_of((size_t)num_buckets, -1);
+    std::vector<LfCellBucket> cells;                       // in bucket (hence partition) order
+    std::vector<int> cell_of((size_t)num_buckets, -1);
     {
         const char* env = getenv("LF_ROW_GROUPS");
         std::vector<int> cand;
@@ -1621,6 +1405,27 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             std::vector<int> chosen;
             for (size_t i = 0; i < cand.size(); ++i)
                 if (h_rg[3 * i + 1] > 0 && h_rg[3 * i] * 100 <= h_rg[3 * i + 1] * kRowGroupMaxPercent) chosen.push_back(cand[i]);
+            // One 16-byte load per lane covers a row of B (256 fp32 or 512 bf16 features): the
+            // chosen buckets are rewritten as cells of rows that are neighbours in up to three
+            // directions where that structure is found, else four consecutive rows at a time.
+            // (fp32 B only: with bf16 the 8 accumulator tiles of a 512-feature row leave room for
+            // one wavefront per SIMD, and the cells measured slower than the row groups)
+            if (!chosen.empty() && lpr == 64 && ch == 1 && b_dtype == LF_DTYPE_F32 && !(env && env[0] == '4')) {
+                std::vector<int> rest;
+                for (int k : chosen) {
+                    LfCellBucket cb{};
+                    bool ok = false;
+                    LF_TRY(lf::cells_build(h_buckets[k], meta[k], num_rows, (int64_t)feat_size * (b_dtype == LF_DTYPE_BF16 ? 2 : 4), s,
+                                           &plan->owned, &plan->temp, &cb, &ok));
+                    if (ok) {
+                        cell_of[k] = (int)cells.size();
+                        cells.push_back(cb);
+                    } else {
+                        rest.push_back(k);
+                    }
+                }
+                chosen.swap(rest);
+            }
             if (!chosen.empty()) {
                 std::vector<int32_t*> m_arrays(chosen.size(), nullptr);
                 for (size_t i = 0; i < chosen.size(); ++i)
@@ -1646,10 +1451,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
                     const int n_blocks = (int)lf::ceil_div(mb.n_groups, 1024);
                     int32_t* partial = nullptr;
                     LF_TRY(dev_alloc(plan, &partial, (size_t)n_blocks + 1, true));
-                    rowgroup_blocksum_kernel<<<n_blocks, 1024, 0, s>>>(m_arrays[i], mb.n_groups, partial);
-                    rowgroup_scanpartial_kernel<<<1, 1024, 0, s>>>(partial, n_blocks);
-                    rowgroup_scan_kernel<<<n_blocks, 1024, 0, s>>>(m_arrays[i], mb.n_groups, partial, n_blocks, goff);
-                    LF_TRY_HIP(hipGetLastError());
+                    LF_TRY_HIP(exclusive_scan_i32(m_arrays[i], mb.n_groups, partial, goff, s));
                     rowgroup_fill_kernel<<<(int)lf::ceil_div(mb.n_groups, 256), 256, 0, s>>>(
                         b.d_cols, b.d_vals, meta[k], b.num_ell_rows, lf::ilog2(b.width), mb.n_groups, goff, ecol, eval, emask);
                     LF_TRY_HIP(hipGetLastError());
@@ -1699,7 +1501,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         for (int k : mine) {
             const lf_bucket_desc& b = h_buckets[k];
             if (b.width > kCoopSlots) continue;            // every row of this bucket is a chunk
-            if (merged_of[k] >= 0) continue;               // served by the row-group kernel
+            if (merged_of[k] >= 0 || cell_of[k] >= 0) continue;   // served by the row-group or the cell kernel
             Group g{};
             g.log_w = lf::ilog2(b.width);
             const int fit = tile_slots(lpr) >> g.log_w;     // ELL rows whose slots fit the LDS tile
@@ -1746,6 +1548,23 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             if (L.merged_begin < 0 || merged_of[k] < L.merged_begin) L.merged_begin = merged_of[k];
             ++L.n_merged;                                  // a partition's buckets are consecutive in `merged`
         }
+        L.cell_begin = -1;
+        for (int k : mine) {
+            if (cell_of[k] < 0) continue;
+            if (L.cell_begin < 0 || cell_of[k] < L.cell_begin) L.cell_begin = cell_of[k];
+            ++L.n_cell_buckets;                            // a partition's buckets are consecutive in `cells`
+        }
+        if (L.n_cell_buckets > 0) {
+            long long longest_c = 0;
+            for (int x = 0; x < kXcds; ++x) {
+                long long len = 0;
+                for (int i = L.cell_begin; i < L.cell_begin + L.n_cell_buckets; ++i)
+                    len += cells[i].n_tiles * (x + 1) / kXcds - cells[i].n_tiles * x / kXcds;
+                longest_c = std::max(longest_c, len);
+            }
+            if (longest_c * kXcds >= (1ll << 31)) return bail(lf::fail(LF_ERR_UNSUPPORTED, "too many cell tiles"));
+            L.cell_grid = (int)(longest_c * kXcds);
+        }
         if (L.n_merged > 0) {
             long long longest_m = 0;
             for (int x = 0; x < kXcds; ++x) {
@@ -1775,6 +1594,10 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         LF_TRY(dev_alloc(plan, &plan->d_merged, merged.size()));
         LF_TRY_HIP(hipMemcpy(plan->d_merged, merged.data(), merged.size() * sizeof(MergedBucket), hipMemcpyHostToDevice));
     }
+    if (!cells.empty()) {
+        LF_TRY(dev_alloc(plan, &plan->d_cells, cells.size()));
+        LF_TRY_HIP(hipMemcpy(plan->d_cells, cells.data(), cells.size() * sizeof(LfCellBucket), hipMemcpyHostToDevice));
+    }
     if (!groups.empty()) {
         LF_TRY(dev_alloc(plan, &plan->d_groups, groups.size()));
         LF_TRY_HIP(hipMemcpy(plan->d_groups, groups.data(), groups.size() * sizeof(Group), hipMemcpyHostToDevice));
@@ -1803,7 +1626,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     plan->info[5] = n_partials;
     plan->info[6] = n_zero;
     (void)occ;
-    plan->info[7] = (int64_t)merged.size();
+    plan->info[7] = (int64_t)(merged.size() + cells.size());
     LF_TRY_HIP(hipStreamSynchronize(s));     // the tables are complete: the plan may run on any stream
     if (free_temporaries(plan) != LF_OK) return bail(lf::fail(LF_ERR_HIP, "hipFree failed on plan-time scratch"));
     *out_plan = plan;
@@ -1832,7 +1655,7 @@ int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t str
     for (int w = 0; w < plan->windows; ++w) {
         for (int p = 0; p < plan->num_parts; ++p) {
             const lf_spmm_plan::Launch& L = plan->launches[p];
-            if (L.n_groups == 0 && L.n_merged == 0) continue;
+            if (L.n_groups == 0 && L.n_merged == 0 && L.n_cell_buckets == 0) continue;
             LaunchArgs a{};
             a.groups = plan->d_groups + L.group_begin;
             a.n_groups = L.n_groups;
@@ -1849,6 +1672,11 @@ int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t str
             if (L.n_merged > 0) {
                 ks.rowgroup<<<L.merged_grid, kWG, 0, s>>>(plan->d_merged + L.merged_begin, L.n_merged, a);
                 LF_HIP(hipGetLastError());
+            }
+            if (L.n_cell_buckets > 0) {
+                if (int rc = lf::cells_launch(plan->d_cells + L.cell_begin, L.n_cell_buckets, L.cell_grid, plan->b_dtype,
+                                              a.B, a.C, a.feat, a.ldb, a.ldc, a.accumulate, s))
+                    return rc;
             }
             if (L.n_heavy > 0) {
                 const int sw = kWG / plan->lpr;

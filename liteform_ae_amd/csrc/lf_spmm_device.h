@@ -1,0 +1,246 @@
+// Device-side building blocks shared by the SpMM kernels of liblfhip.so: launch arguments,
+// dense-operand access (one 16-byte load per lane), per-lane accumulators, row stores.
+// Everything lives in an anonymous namespace: each translation unit gets its own copy.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "lf_internal.h"
+
+namespace {
+
+constexpr int kWG = 256;            // threads per workgroup (4 wavefronts)
+#ifndef LF_TILE_SLOTS_PER_SUBWAVE
+#define LF_TILE_SLOTS_PER_SUBWAVE 64
+#endif
+#ifndef LF_UNROLL
+#define LF_UNROLL 8
+#endif
+#ifndef LF_TILE_MIN
+#define LF_TILE_MIN 512
+#endif
+// (col, val) pairs staged in LDS per tile: a fixed amount of work per sub-wave, so narrow
+// feature sizes (many sub-waves per workgroup) get larger tiles.  N = 128 -> 512 slots.
+constexpr int tile_slots(int lpr) {
+    const int n = LF_TILE_SLOTS_PER_SUBWAVE * (kWG / lpr);
+    return n < LF_TILE_MIN ? LF_TILE_MIN : n;
+}
+constexpr int kTileRows = 512;      // ELL rows per tile at most (<= tile_slots)
+#ifndef LF_COOP_SLOTS
+#define LF_COOP_SLOTS 256
+#endif
+#ifndef LF_CHUNK_SLOTS
+#define LF_CHUNK_SLOTS 2048
+#endif
+constexpr int kCoopSlots = LF_COOP_SLOTS;    // a source row with more slab slots is reduced by a whole workgroup
+constexpr int kChunkSlots = LF_CHUNK_SLOTS;  // ... in chunks of this many slots (a whole number of ELL rows)
+constexpr int kXcds = 8;
+constexpr int kPartBytesMax = 16384;   // LDS for per-ELL-row sums of a balanced segment tile at most
+constexpr int kUnroll = LF_UNROLL;  // B-row gathers in flight per sub-wave
+constexpr uint32_t kMetaLenMask = 0x7FFu;
+constexpr int kMetaLenBits = 11;
+
+enum GroupType : int { kEll = 0, kSeg = 1, kZero = 2, kChunk = 3, kEllSeg = 4 };
+
+struct Chunk {
+    long long slot_begin;   // first slot, relative to the bucket's slab
+    int n_slots;
+    int partial;            // index of the partial row this chunk produces; < 0: the chunk is the
+                            // whole source row and goes straight to C
+    int row;                // source row
+    int pad_;
+};
+
+struct HeavyRow {
+    int row;
+    int partial_begin;
+    int n_partials;
+    int pad_;
+};
+
+struct Group {
+    int type;
+    int log_w;
+    int rows_per_tile;
+    int balanced;                 // kEllSeg: per-ELL-row sums through LDS (needs rows_per_tile * N floats)
+    long long n_items;            // ELL rows / rows to clear / chunks
+    long long n_tiles;
+    const int32_t* rows;          // kEll, kSeg: source rows; kZero: rows to clear
+    const int32_t* meta;
+    const int32_t* cols;
+    const float* vals;
+    const Chunk* chunks;          // kChunk
+};
+
+struct LaunchArgs {
+    const Group* groups;
+    int n_groups;
+    int accumulate;               // 0: C = result, 1: C += result
+    int feat;                     // N: features computed by the launch
+    int ldb, ldc;                 // row strides of B and C in elements (N, or more for a feature window)
+    int pad_;
+    const void* B;
+    float* C;
+    float* partials;
+};
+
+// ------------------------------------------------------------------------------------
+// Dense-operand access: VEC features per lane as one 16-byte load.
+template <typename BT> struct Dense;
+
+template <> struct Dense<float> {
+    static constexpr int kVec = 4;
+    __device__ static __forceinline__ void load(const void* B, size_t elem, float (&x)[4]) {
+        const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(B) + elem);
+        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    }
+};
+
+struct bf16_t { uint16_t bits; };
+
+template <> struct Dense<bf16_t> {
+    static constexpr int kVec = 8;
+    __device__ static __forceinline__ void load(const void* B, size_t elem, float (&x)[8]) {
+        const uint4 v = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(B) + elem);
+        x[0] = __uint_as_float(v.x << 16); x[1] = __uint_as_float(v.x & 0xFFFF0000u);
+        x[2] = __uint_as_float(v.y << 16); x[3] = __uint_as_float(v.y & 0xFFFF0000u);
+        x[4] = __uint_as_float(v.z << 16); x[5] = __uint_as_float(v.z & 0xFFFF0000u);
+        x[6] = __uint_as_float(v.w << 16); x[7] = __uint_as_float(v.w & 0xFFFF0000u);
+    }
+};
+
+// Accumulator of one sub-wave lane: CH chunks of VEC features.
+template <int CH, int VEC> struct Acc {
+    float v[CH][VEC];
+    __device__ __forceinline__ void clear() {
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) v[c][i] = 0.f;
+    }
+};
+
+// Position of a lane inside the feature dimension.
+template <int LPR, int CH, int VEC> struct Lane {
+    int sl;                 // lane inside the sub-wave
+    int feat;               // N: features this launch computes
+    int ldb, ldc;           // elements between consecutive rows of B and of C (>= N)
+    int f[CH];              // first feature of each chunk (clamped to 0 when outside N)
+    bool on[CH];
+    __device__ __forceinline__ Lane(int sl_, int feat_, int ldb_, int ldc_)
+        : sl(sl_), feat(feat_), ldb(ldb_), ldc(ldc_) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int f0 = (c * LPR + sl_) * VEC;
+            on[c] = f0 < feat_;
+            f[c] = on[c] ? f0 : 0;
+        }
+    }
+};
+
+template <int U, int LPR, int CH, typename BT>
+__device__ __forceinline__ void gather_fma(const void* B, const Lane<LPR, CH, Dense<BT>::kVec>& ln,
+                                           const int (&col)[U], const float (&val)[U],
+                                           Acc<CH, Dense<BT>::kVec>& acc) {
+    constexpr int VEC = Dense<BT>::kVec;
+    float x[U][CH][VEC];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+            Dense<BT>::load(B, (size_t)(uint32_t)col[u] * (size_t)ln.ldb + ln.f[c], x[u][c]);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc.v[c][i] = fmaf(val[u], x[u][c][i], acc.v[c][i]);
+}
+
+template <int LPR, int CH, int VEC>
+__device__ __forceinline__ void store_row(float* C, int row, const Lane<LPR, CH, VEC>& ln,
+                                          const Acc<CH, VEC>& acc, int accumulate) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        if (!ln.on[c]) continue;
+        float* dst = C + (size_t)row * ln.ldc + ln.f[c];
+#pragma unroll
+        for (int i = 0; i < VEC; i += 4) {
+            float4 o = make_float4(acc.v[c][i], acc.v[c][i + 1], acc.v[c][i + 2], acc.v[c][i + 3]);
+            if (accumulate) {
+                const float4 old = *reinterpret_cast<const float4*>(dst + i);
+                o.x += old.x; o.y += old.y; o.z += old.z; o.w += old.w;
+            }
+            *reinterpret_cast<float4*>(dst + i) = o;
+        }
+    }
+}
+
+// goff[g] = exclusive prefix of m[g], goff[n_groups] = total, in three small launches:
+// sums of blocks of 1024 groups, their exclusive scan by one workgroup (in place, total
+// appended), then the scan inside every block.
+__device__ __forceinline__ int block_inclusive_scan_1024(int x, int* s_wave) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl = x;
+    for (int d = 1; d < 64; d <<= 1) {
+        const int y = __shfl_up(incl, d);
+        if (lane >= d) incl += y;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) incl += s_wave[w];
+    __syncthreads();
+    return incl;
+}
+
+__global__ void __launch_bounds__(1024)
+scan_blocksum_kernel(const int32_t* __restrict__ m, long long n_groups, int32_t* __restrict__ partial) {
+    __shared__ int s_wave[16];
+    const long long i = (long long)blockIdx.x * 1024 + threadIdx.x;
+    const int incl = block_inclusive_scan_1024(i < n_groups ? m[i] : 0, s_wave);
+    if (threadIdx.x == 1023) partial[blockIdx.x] = incl;
+}
+
+__global__ void __launch_bounds__(1024)
+scan_partials_kernel(int32_t* __restrict__ partial, int n_blocks) {
+    __shared__ int s_wave[16];
+    __shared__ int s_carry;
+    if (threadIdx.x == 0) s_carry = 0;
+    __syncthreads();
+    for (int base = 0; base < n_blocks; base += 1024) {
+        const int i = base + threadIdx.x;
+        const int x = i < n_blocks ? partial[i] : 0;
+        const int incl = block_inclusive_scan_1024(x, s_wave);
+        const int carry = s_carry;
+        if (i < n_blocks) partial[i] = carry + incl - x;
+        __syncthreads();
+        if (threadIdx.x == 1023) s_carry = carry + incl;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) partial[n_blocks] = s_carry;
+}
+
+__global__ void __launch_bounds__(1024)
+scan_blocks_kernel(const int32_t* __restrict__ m, long long n_groups, const int32_t* __restrict__ partial,
+                     int n_blocks, int32_t* __restrict__ goff) {
+    __shared__ int s_wave[16];
+    const long long i = (long long)blockIdx.x * 1024 + threadIdx.x;
+    const int x = i < n_groups ? m[i] : 0;
+    const int incl = block_inclusive_scan_1024(x, s_wave);
+    if (i < n_groups) goff[i] = partial[blockIdx.x] + incl - x;
+    if (blockIdx.x == 0 && threadIdx.x == 0) goff[n_groups] = partial[n_blocks];
+}
+
+// off[i] = exclusive prefix of m[i] for i < n, off[n] = total, enqueued on `s`.  `partial`
+// needs ceil(n / 1024) + 1 ints.
+inline hipError_t exclusive_scan_i32(const int32_t* m, long long n, int32_t* partial, int32_t* off, hipStream_t s) {
+    const int n_blocks = (int)((n + 1023) / 1024);
+    if (n_blocks == 0) return hipSuccess;
+    scan_blocksum_kernel<<<n_blocks, 1024, 0, s>>>(m, n, partial);
+    scan_partials_kernel<<<1, 1024, 0, s>>>(partial, n_blocks);
+    scan_blocks_kernel<<<n_blocks, 1024, 0, s>>>(m, n, partial, n_blocks, off);
+    return hipGetLastError();
+}
+
+}  // namespace
