@@ -11,11 +11,13 @@ configuration the headline metric is quoted on.  Prints one JSON line:
   roofline         HBM: algorithmic bytes per step / average kernel time of a step measured
                    with HIP events on the launch stream (a step is one launch per column
                    partition and feature window; bytes and time are both summed over them, so
-                   the ratio is also the per-launch one); traffic = L2<->fabric bytes per step from rocprofv3
-                   counters when a measurement is on file
-  format_compose   bucket-width search and slab build times (GPU), reported beside it
+                   the ratio is also the per-launch one); traffic = L2<->fabric bytes per step from
+                   the rocprofv3 counter runs on file for exactly these kernel sources, else null
+  format_compose   launch-shape choice, bucket-width search, slab build and kernel plan times
+                   (GPU), their sum with the upload as end_to_end_ms, and the same search and
+                   build through the CPU restatement on the two small workloads
   cpu_baseline     scipy CSR @ dense (the reference's own CPU product, one thread) on a
-                   bounded sample of rows of the same matrix
+                   bounded sample of rows of the same matrix, 1 warm-up + median of 3
 """
 from __future__ import annotations
 
@@ -44,30 +46,52 @@ def gather_bytes(nnz, rows, feat, b_bytes):
     return nnz * 8 + (rows + 1) * 4 + nnz * feat * b_bytes + rows * feat * 4
 
 
-# L2 <-> fabric bytes per step (all launches of a step; /W2 = two feature windows) from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE, FETCH_SIZE scaled by 2.000 as calibrated on a 1 GiB copy in the same runs;
-# source: profiles/spmm_partition_kernel.cfg3_N128.md
-MEASURED_TRAFFIC = {
-    "cfg3/N128/P1": 44157630417,
-    "cfg3/N128/P2": 46512630501,
-    "cfg3/N128/P3": 48665180588,
-    "cfg3/N128/P1/W2": 45234112102,
-    "cfg3/N128/P2/W2": 47336937882,
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.md")
+KERNEL_SOURCES = ("lf_spmm.hip", "lf_cells.hip", "lf_spmm_device.h")
+
+
+def kernel_source_id():
+    """git blob ids (sha1 of "blob <size>\\0<content>") of the SpMM kernel sources, joined: what a
+    counter measurement on file has to name to be reported for this build."""
+    import hashlib
+    ids = []
+    for name in KERNEL_SOURCES:
+        data = open(os.path.join(ROOT, "liteform_ae_amd", "csrc", name), "rb").read()
+        ids.append(hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest()[:12])
+    return "+".join(ids)
 
 
 def recorded_traffic(workload, feat, parts, windows):
-    return MEASURED_TRAFFIC.get(f"{workload}/N{feat}/P{parts}" + (f"/W{windows}" if windows > 1 else ""))
+    """L2 <-> fabric bytes per step from the rocprofv3 counter runs summarised in
+    profiles/hbm_traffic.md (FETCH_SIZE and WRITE_SIZE, calibrated on a plain copy).  A row
+    counts only if it was taken with the kernel sources of this build (their git blob ids are
+    in the row); otherwise the figure is unknown and reported as null."""
+    key = f"{workload}/N{feat}/P{parts}/W{windows}"
+    try:
+        lines = open(TRAFFIC_FILE).read().splitlines()
+    except OSError:
+        return None
+    here = kernel_source_id()
+    for line in lines:
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 4 and cells[0] == key and cells[3] == here:
+            try:
+                return int(cells[2].replace(",", ""))
+            except ValueError:
+                return None
+    return None
 
 
 def cpu_baseline(wl, B_host, feat, budget_s=20.0):
-    """scipy CSR(f32) @ dense(f32) on the first rows of the matrix, sized to ~budget_s."""
+    """scipy CSR(f32) @ dense(f32) - the reference's own CPU product, one thread - on the first
+    rows of the matrix: one warm-up and three timed runs, sized so that the four together take
+    about budget_s; the median is reported."""
     import scipy.sparse as sp
     indptr, indices, data = wl.matrix.adj_tensors("csr")
     rows = wl.shape[0]
     nnz = int(indptr[-1])
-    # ~1 GFLOP/s is typical for scipy's single-threaded csr_matvecs at this width
-    target_nnz = int(budget_s * 1.0e9 / (2 * feat))
+    # ~3 GFLOP/s is typical for scipy's single-threaded csr_matvecs at this width
+    target_nnz = int(budget_s / 4 * 3.0e9 / (2 * feat))
     if nnz <= target_nnz:
         take = rows
     else:
@@ -77,16 +101,20 @@ def cpu_baseline(wl, B_host, feat, budget_s=20.0):
     A = sp.csr_matrix((np.asarray(data[:sub_nnz], dtype=np.float32), indices[:sub_nnz], indptr[:take + 1]),
                       shape=(take, wl.shape[1]))
     Bf = np.ascontiguousarray(B_host, dtype=np.float32)
-    t0 = time.perf_counter()
-    out = A @ Bf
-    dt = time.perf_counter() - t0
+    out = A @ Bf                                            # warm-up
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        out = A @ Bf
+        times.append(time.perf_counter() - t0)
+    dt = float(np.median(times))
     res = {
         "value": round(2.0 * sub_nnz * feat / dt / 1e9, 3),
         "unit": "GFLOP/s",
         "cores": 1,
         "kind": "port",
         "sample": f"scipy csr_matrix(f32) @ dense(f32), first {take} of {rows} rows "
-                  f"({sub_nnz} nnz), 1 run, {dt:.2f} s",
+                  f"({sub_nnz} nnz), 1 warm-up + median of 3 runs, {dt:.2f} s each",
     }
     # the same sample through torch's threaded CPU CSR product, as a multi-core figure
     try:
@@ -111,6 +139,40 @@ def cpu_baseline(wl, B_host, feat, budget_s=20.0):
     except Exception as exc:                                # a baseline only: report, do not fail the bench
         res["threaded"] = {"value": None, "error": f"{type(exc).__name__}: {exc}"}
     return res, out, take
+
+
+def compose_cpu_baseline(fa, make_workload, cost_model):
+    """Format composition on the CPU beside the GPU, on the two workloads the CPU restatement
+    finishes in seconds: the oracle's search_bucket_config (the reference's pure-Python
+    algorithm: what its driver times as time_bucket) and its closed-form numpy builder, against
+    search + slab build through the library on the same matrices.  Beyond these sizes the
+    Python search takes minutes: not run, never extrapolated."""
+    from oracle import liteform_oracle as O
+    out = {}
+    for name in ("cfg1", "cfg2"):
+        wl = make_workload(name)
+        g, parts, feat = wl.matrix, wl.num_parts or 1, wl.feat_size
+        t0 = time.perf_counter()
+        want = O.search_bucket_config(g, parts, O.OracleCostModelSettings(feat, parts))
+        cpu_search = (time.perf_counter() - t0) * 1e3
+        t0 = time.perf_counter()
+        O.build_hyb_format_closed_form(g, want)
+        cpu_build = (time.perf_counter() - t0) * 1e3
+        cfg_obj = fa.CostModelSettings(feat, parts, cost_model="reference")
+        fa.search_bucket_config(g, parts, cfg_obj)          # warm (uploads the matrix)
+        t0 = time.perf_counter()
+        got = fa.search_bucket_config(g, parts, cfg_obj)
+        gpu_search = (time.perf_counter() - t0) * 1e3
+        fa.build_hyb_format_device(g, got)
+        t0 = time.perf_counter()
+        fa.build_hyb_format_device(g, got)
+        gpu_build = (time.perf_counter() - t0) * 1e3
+        out[name] = {"nnz": wl.nnz, "num_parts": parts, "same_config": got == want,
+                     "cpu_search_ms": round(cpu_search, 2), "cpu_build_ms": round(cpu_build, 2),
+                     "gpu_search_ms": round(gpu_search, 3), "gpu_build_ms": round(gpu_build, 3)}
+    out["note"] = ("cpu = oracle/liteform_oracle.py (pure-Python search, numpy closed-form builder), 1 core; "
+                   "reference cost model on both sides; cfg3-cfg5: not run (the Python search takes minutes)")
+    return out
 
 
 def bench_bsr(args):
@@ -179,9 +241,12 @@ def main():
     ap.add_argument("--workload", default="cfg3")
     ap.add_argument("--feat", type=int, default=0, help="dense columns N (default: the workload's)")
     ap.add_argument("--parts", type=int, default=0,
-                    help="column partitions (default: the workload's; measured choice where it names none)")
+                    help="column partitions (default: the workload's; chosen by --shape where it names none)")
     ap.add_argument("--windows", type=int, default=0,
-                    help="feature windows per step (0 = by measurement together with the partitions)")
+                    help="feature windows per step (0 = chosen together with the partitions)")
+    ap.add_argument("--shape", default="model", choices=["model", "measured"],
+                    help="how an open partition / window count is chosen: the launch-shape model "
+                         "(default) or by composing and timing the candidates")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the matrix (testing only)")
     ap.add_argument("--b-dtype", default="", choices=["", "f32", "bf16"], help="dtype of B (default: the workload's)")
     ap.add_argument("--cost-model", default="gfx950", choices=["reference", "gfx950"],
@@ -240,14 +305,28 @@ def main():
     ingest_ms = (time.perf_counter() - t0) * 1e3
     part_timings = None
     windows = args.windows
-    if not parts or not windows:            # left open: partition count and feature windows by measurement
-        t0 = time.perf_counter()
-        (parts, windows), shape_timings = fa.choose_launch_shape(
-            g, feat, wl.b_dtype, candidates=(parts,) if parts else (1, 2, 3, 4),
-            windows=(windows,) if windows else None, cost_model=args.cost_model, return_timings=True)
-        part_timings = {f"P{p}xW{w}": round(t, 4) for (p, w), t in shape_timings.items()}
-        print(f"[bench] launch shape chosen by measurement: {parts} partition(s) x {windows} feature window(s) "
-              f"from {part_timings} ({time.perf_counter() - t0:.2f} s)", file=sys.stderr, flush=True)
+    shape_ms = 0.0
+    shape_how = "given"
+    if not parts or not windows:            # left open: partition count and feature windows
+        cands = (parts,) if parts else (1, 2, 3, 4)
+        wins = (windows,) if windows else None
+        if args.shape == "model":
+            fa.predict_launch_shape(g, feat, wl.b_dtype, candidates=cands, windows=wins)          # warm
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            (parts, windows), table = fa.predict_launch_shape(g, feat, wl.b_dtype, candidates=cands, windows=wins,
+                                                              return_predictions=True)
+            shape_ms = (time.perf_counter() - t0) * 1e3
+            shape_how = "model"
+        else:
+            t0 = time.perf_counter()
+            (parts, windows), table = fa.choose_launch_shape(g, feat, wl.b_dtype, candidates=cands, windows=wins,
+                                                             cost_model=args.cost_model, return_timings=True)
+            shape_ms = (time.perf_counter() - t0) * 1e3
+            shape_how = "measured"
+        part_timings = {f"P{p}xW{w}": round(t, 4) for (p, w), t in table.items()}
+        print(f"[bench] launch shape ({shape_how}): {parts} partition(s) x {windows} feature window(s) "
+              f"from {part_timings or 'the row-overlap rule'} ({shape_ms:.2f} ms)", file=sys.stderr, flush=True)
     cfg_obj = fa.CostModelSettings(feat, parts, cost_model=args.cost_model)
     fa.search_bucket_config(g, parts, cfg_obj)            # warm
     t0 = time.perf_counter()
@@ -301,7 +380,7 @@ def main():
     algo = algorithmic_bytes(nnz, rows, cols, feat, b_bytes)
     gath = gather_bytes(nnz, rows, feat, b_bytes)
     achieved = algo / (kernel_ms * 1e-3) / 1e9
-    traffic = recorded_traffic(wl.name if args.scale == 1.0 else "", feat, parts, windows)
+    traffic = recorded_traffic(wl.name if args.scale == 1.0 and not args.widths else "", feat, parts, windows)
 
     result = {
         "metric": "SpMM GFLOP/s & % HBM roofline at N=128; format-compose ms",
@@ -320,6 +399,7 @@ def main():
             "workload": f"{wl.name}: {wl.description}" + ("" if args.scale == 1.0 else f" (scale {args.scale})"),
             "rows": rows, "cols": cols, "nnz": nnz, "feat_size": feat, "num_parts": parts, "feature_windows": windows,
             "bucket_widths": config, "cost_model": args.cost_model,
+            "launch_shape": shape_how,
             "launch_shape_candidates_ms": part_timings,
         },
         "roofline": {
@@ -329,6 +409,8 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 5),
             "traffic": traffic,
+            "traffic_source": "profiles/hbm_traffic.md" if traffic is not None else None,
+            "kernel_source_id": kernel_source_id(),
             "launches_per_step": parts * windows,
             "kernel_ms": round(kernel_ms, 4),
             "kernel_ms_median": round(float(np.median(ev_ms)), 4),
@@ -343,13 +425,17 @@ def main():
             "build_ms": round(build_ms, 3),
             "total_ms": round(search_ms + build_ms, 3),
             "kernel_plan_ms": round(plan_ms, 3),        # tile tables of the fused kernel (the reference: TVM build)
+            "launch_shape_ms": round(shape_ms, 3),      # choosing partitions x windows (model, or measurement)
             "coo_upload_and_csr_ms": round(ingest_ms, 1),
+            # everything between "matrix on the host" and "first product can start"
+            "end_to_end_ms": round(ingest_ms + shape_ms + search_ms + build_ms + plan_ms, 2),
             "slab_slots": fmt.total_slots(),
             "ell_rows": int(np.sum(fmt.ell_rows)),
         },
     }
 
     if not args.no_cpu:
+        result["format_compose"]["cpu_baseline"] = compose_cpu_baseline(fa, make_workload, args.cost_model)
         base, ref_rows, take = cpu_baseline(wl, B_host, feat, args.cpu_seconds)
         base["host_cpus"] = os.cpu_count()
         result["cpu_baseline"] = base

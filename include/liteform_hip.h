@@ -53,7 +53,7 @@ extern "C" {
 #define LF_DTYPE_BF16 1
 
 #define LF_COST_REFERENCE 0     /* format_algos.py:1035-1166 bit for bit */
-#define LF_COST_GFX950 1        /* traffic model for MI355X; same search, different cost */
+#define LF_COST_GFX950 1        /* measured cost of ELL rows, staged slots and slab bytes on MI355X; same search */
 
 typedef void* lf_stream_t;
 typedef struct lf_spmm_plan lf_spmm_plan;
@@ -139,6 +139,27 @@ int lf_search_bucket_config(const int64_t* h_stats, const int64_t* h_colhist, in
                             int32_t width_limit, int32_t cfg_feat_size, int32_t cfg_num_parts,
                             int32_t cost_model, int32_t* h_widths, int32_t* h_nwidths,
                             double* h_trace_cost, int32_t* h_trace_len);
+
+/* Launch shape without running the kernel: the predicted time in milliseconds of one product
+ * with num_parts column partitions (h_stats: their bucket statistics from lf_bucket_stats,
+ * [num_parts][LF_MAX_CLASSES][LF_STATS_FIELDS]) and n_windows feature windows
+ * (lf_spmm_set_windows), for a matrix whose rows do not share columns (scattered gathers).
+ * Stands where the reference predicts num_parts from matrix features with a trained model
+ * (proc05.spmm.end-to-end.py:82-97, 142): the caller evaluates the candidates and takes the
+ * cheapest.  The model prices the gathers, the read-modify-write of C by later partitions and
+ * the slabs against the fabric rate and the scattered-row HBM rate of MI355X, with the share of
+ * B that the 256 MB memory-side cache holds.  Host only. */
+int lf_model_spmm_ms(const int64_t* h_stats, int32_t num_parts, int32_t n_windows, int64_t num_rows,
+                     int64_t num_cols, int32_t feat_size, int32_t b_dtype, double* h_ms);
+
+/* Share of the entries of every sample_stride-th row whose column also occurs in the row
+ * before it: h_out = {entries in both rows, entries looked at}.  Near 0 for matrices with
+ * scattered columns, 0.67 for a 27-point stencil; rows that share columns read B through the
+ * L2 and gain nothing from column partitions or feature windows.  d_scratch: 16 bytes of
+ * device memory.  Synchronises the stream.  (One of the inputs of the launch-shape choice, as
+ * MTX.matrix_features, format_matrix_market.py:153-202, is of the reference's predictor.) */
+int lf_row_overlap(const int32_t* d_indptr, const int32_t* d_indices, int64_t num_rows, int64_t sample_stride,
+                   void* d_scratch, int64_t* h_out /* [2] */, lf_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
  * hyb composition.  Replaces build_hyb_format (format_algos.py:226-385).

@@ -56,6 +56,8 @@ SIGNATURES = {
     "lf_row_features_static": (C.c_int, [vp, C.c_int64, vp, vp]),
     "lf_search_bucket_config": (C.c_int, [i64p, i64p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                           i32p, i32p, f64p, i32p]),
+    "lf_model_spmm_ms": (C.c_int, [i64p, C.c_int32, C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, f64p]),
+    "lf_row_overlap": (C.c_int, [vp, vp, C.c_int64, C.c_int64, vp, vp, vp]),
     "lf_hyb_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int32, C.c_int32]),
     "lf_hyb_layout": (C.c_int, [i64p, i32p, C.c_int32, i64p, i64p, i64p, i64p]),
     "lf_stats_seg_bounds": (vp, [vp, C.c_int64, C.c_int32]),

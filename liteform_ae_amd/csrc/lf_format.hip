@@ -148,6 +148,35 @@ row_features_kernel(const int32_t* __restrict__ indptr, int64_t rows, unsigned l
     }
 }
 
+// out[0] += entries of row r that also occur in row r - 1, out[1] += entries of row r, for every
+// stride-th row r >= 1 (two-pointer walk over the two ascending column lists)
+__global__ void __launch_bounds__(kBlock)
+row_overlap_kernel(const int32_t* __restrict__ indptr, const int32_t* __restrict__ indices, int64_t rows,
+                   int64_t stride, unsigned long long* __restrict__ out) {
+    unsigned long long both = 0, seen = 0;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t r = 1 + i * stride;
+        if (r >= rows) break;
+        int a = indptr[r - 1], b = indptr[r];
+        const int a_end = b, b_end = indptr[r + 1];
+        seen += (unsigned long long)(b_end - b);
+        while (a < a_end && b < b_end) {
+            const int ca = indices[a], cb = indices[b];
+            both += ca == cb;
+            a += ca <= cb;
+            b += cb <= ca;
+        }
+    }
+    for (int d = 32; d > 0; d >>= 1) {
+        both += __shfl_xor(both, d);
+        seen += __shfl_xor(seen, d);
+    }
+    if ((threadIdx.x & 63) == 0 && seen) {
+        atomicAdd(&out[0], both);
+        atomicAdd(&out[1], seen);
+    }
+}
+
 // Initial width class of a segment of `deg` entries: width = min(next_pow2(deg), limit),
 // cost-model rows = max(1, next_pow2(deg) / limit)            (format_algos.py:875-882)
 __device__ __forceinline__ void width_class(int deg, int kmax, int& k, int& cost_rows) {
@@ -771,6 +800,26 @@ int lf_row_features(const int32_t* d_indptr, int64_t num_rows, void* d_scratch, 
     row_features_kernel<<<grid, kBlock, 0, s>>>(d_indptr, num_rows, acc);
     LF_HIP(hipGetLastError());
     LF_HIP(hipMemcpyAsync(h_out, acc, 32, hipMemcpyDeviceToHost, s));
+    LF_HIP(hipStreamSynchronize(s));
+    return LF_OK;
+}
+
+int lf_row_overlap(const int32_t* d_indptr, const int32_t* d_indices, int64_t num_rows, int64_t sample_stride,
+                   void* d_scratch, int64_t* h_out, lf_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    LF_REQUIRE(h_out, LF_ERR_INVALID, "h_out is null");
+    LF_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31) && sample_stride >= 1, LF_ERR_INVALID, "bad num_rows / stride");
+    h_out[0] = h_out[1] = 0;
+    if (num_rows < 2) return LF_OK;
+    LF_REQUIRE(d_indptr && d_indices && d_scratch, LF_ERR_INVALID, "null argument");
+    LF_REQUIRE((uintptr_t)d_scratch % 8 == 0, LF_ERR_INVALID, "scratch must be 8-byte aligned");
+    unsigned long long* acc = (unsigned long long*)d_scratch;
+    LF_HIP(fill_u32(acc, 4, 0u, s));
+    const int64_t samples = (num_rows - 1 + sample_stride - 1) / sample_stride;
+    const int grid = (int)std::min<int64_t>((samples + kBlock - 1) / kBlock, 1024);
+    row_overlap_kernel<<<grid, kBlock, 0, s>>>(d_indptr, d_indices, num_rows, sample_stride, acc);
+    LF_HIP(hipGetLastError());
+    LF_HIP(hipMemcpyAsync(h_out, acc, 16, hipMemcpyDeviceToHost, s));
     LF_HIP(hipStreamSynchronize(s));
     return LF_OK;
 }

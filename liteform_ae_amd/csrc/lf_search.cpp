@@ -15,6 +15,7 @@
 // This file must be compiled without floating-point contraction (-ffp-contract=off) so the
 // double arithmetic matches CPython's operation by operation.
 #include <algorithm>
+#include <cmath>
 #include <cstring>
 #include <vector>
 
@@ -104,34 +105,57 @@ double reference_cost(const Pool& pool, const int64_t* hist, int nmask, int32_t 
     return cost;
 }
 
-// Cost of a state for the gfx950 kernels, in bytes of HBM-traffic equivalent.  The B gather
-// (nnz * feat * sizeof(B)) and the C store are the same for every state of the fold chain, so
-// only what a fold changes is priced:
-//   * 8 bytes per slab slot (column + value are streamed once, padding included);
-//   * kRowBytes per ELL row: 8 bytes of row id + meta, and the fixed work of starting a row
-//     (descriptor reads, loop set-up, a sub-wave slot left idle on continuation rows).
-// kRowBytes was fitted on MI355X: on the 2.45M-row power-law graph at N = 128 every extra
-// million ELL rows costs 0.07-0.2 ms at ~6 TB/s, i.e. 400-1200 bytes each, while padded slots
-// cost no more than their slab bytes because a padded slot re-reads a row that is already
-// in flight.  With these weights a fold pays only when it removes far more padding than it
-// adds rows, which on the benchmark workloads keeps the initial power-of-two widths.
-constexpr double kSlotBytes = 8.0;
-constexpr double kRowBytes = 600.0;
+// ---------------------------------------------------------------------------------------
+// gfx950 model.  All constants below were measured on MI355X with this library's kernels
+// (2.45M-row power-law graph, 500k x 2M skewed matrix, uniform-degree matrices of 17 / 33 /
+// 130 / 520 entries per row; N = 32 .. 512, 1-4 column partitions, 1-8 feature windows).
+//
+// Fold chain.  The kernels walk only the valid slots of an ELL row (rounded up to the unroll
+// of eight), so padding costs no gathers; what a state changes is
+//   * the slots that are read and staged through LDS whole, padding included (buckets of up
+//     to 64 slots; wider rows are streamed and only their valid slots are touched):
+//     8 bytes per slot at the fabric rate plus kStagedSlotPs;
+//   * the number of ELL rows - row id and meta, loop set-up, one store (or partial sum) per
+//     row: row_ps(N) per row, dearer at small N where many short rows share a wavefront.
+// A class folded into a narrower bucket takes ceil(average fill / width) ELL rows per source
+// row.  Measured against this model: folding never gains more than 3 % (33 entries per row,
+// N = 128: widths [16] 2.32 ms against [64] 2.38 ms, which the model reproduces), and the
+// power-law and skewed benchmark matrices keep their initial power-of-two widths.
+constexpr double kFabricBytesPerPs = 7.493;       // 7.49 TB/s: what the fabric moves at best
+constexpr double kStagedSlotPs = 6.7;
+constexpr int kStagedWidthMax = 64;
 
-double gfx950_cost(const Pool& pool, const int64_t* hist, int nmask, int32_t feat, int32_t parts) {
-    (void)hist;
-    (void)nmask;
-    (void)feat;
-    (void)parts;
-    double cost = 0.0;
-    for (const Bucket& b : pool.items)
-        cost += kSlotBytes * (double)b.num_rows * (double)b.width + kRowBytes * (double)b.num_rows;
-    return cost;
+double row_ps(int feat) {
+    if (feat <= 32) return 230.0;
+    if (feat <= 64) return 70.0;
+    if (feat <= 128) return 40.0;
+    if (feat <= 256) return 60.0;
+    return 90.0;
 }
 
-double state_cost(int model, const Pool& pool, const int64_t* hist, int nmask, int32_t feat, int32_t parts) {
-    return model == LF_COST_GFX950 ? gfx950_cost(pool, hist, nmask, feat, parts)
-                                   : reference_cost(pool, hist, nmask, feat, parts);
+// st: this partition's initial statistics [LF_MAX_CLASSES][LF_STATS_FIELDS]
+double gfx950_cost(const Pool& pool, const int64_t* st, int32_t feat) {
+    double ps = 0.0;
+    for (const Bucket& b : pool.items) {
+        for (int k = 0; k < LF_MAX_CLASSES; ++k) {
+            if (!(b.classes >> k & 1u)) continue;
+            const double rows = (double)st[(size_t)k * LF_STATS_FIELDS + 2];
+            const double nnz = (double)st[(size_t)k * LF_STATS_FIELDS + 1];
+            if (rows <= 0) continue;
+            const double per_row = std::ceil(nnz / rows / (double)b.width);
+            const double ell = rows * std::max(1.0, per_row);
+            const double slots = ell * (double)b.width;
+            ps += ell * row_ps(feat);
+            // wider rows are streamed: only their valid slots are read, the same in every state
+            if (b.width <= kStagedWidthMax) ps += slots * (kStagedSlotPs + 8.0 / kFabricBytesPerPs);
+        }
+    }
+    return ps;
+}
+
+double state_cost(int model, const Pool& pool, const int64_t* hist, int nmask, const int64_t* st, int32_t feat,
+                  int32_t parts) {
+    return model == LF_COST_GFX950 ? gfx950_cost(pool, st, feat) : reference_cost(pool, hist, nmask, feat, parts);
 }
 
 }  // namespace
@@ -194,7 +218,7 @@ extern "C" int lf_search_bucket_config(const int64_t* h_stats, const int64_t* h_
         }
 
         // modify_bucket_widths (format_algos.py:727-774)
-        double best_cost = state_cost(cost_model, pool, hist, nmask, cfg_feat_size, cfg_num_parts);
+        double best_cost = state_cost(cost_model, pool, hist, nmask, st, cfg_feat_size, cfg_num_parts);
         std::vector<int32_t> best = pool.sorted_widths();
         if (trace) trace[ntrace] = best_cost;
         ++ntrace;
@@ -202,7 +226,7 @@ extern "C" int lf_search_bucket_config(const int64_t* h_stats, const int64_t* h_
         int32_t neww = pre / 2;
         while (neww >= 1) {
             move_largest_bucket(pool, pre, neww);
-            const double c = state_cost(cost_model, pool, hist, nmask, cfg_feat_size, cfg_num_parts);
+            const double c = state_cost(cost_model, pool, hist, nmask, st, cfg_feat_size, cfg_num_parts);
             if (trace) trace[ntrace] = c;
             ++ntrace;
             if (c < best_cost) {
@@ -216,5 +240,67 @@ extern "C" int lf_search_bucket_config(const int64_t* h_stats, const int64_t* h_
         for (size_t i = 0; i < best.size(); ++i) out_w[i] = best[i];
         if (h_trace_len) h_trace_len[p] = ntrace;
     }
+    return LF_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// Launch shape.  Predicted time of one product with `num_parts` column partitions and
+// `n_windows` feature windows, from the partitions' bucket statistics alone.
+//
+// One launch (one partition, one window of n = feat / windows features) moves
+//   gathers  nnz_p rows of g = n * sizeof(B) bytes each,
+//   C        rows * n * 4 bytes written by partition 0, 8 bytes per feature and touched row
+//            (read-modify-write) by every later partition,
+//   slabs    8 bytes per slot and per ELL row.
+// Everything crosses the fabric, which moves kFabricBytesPerPs at best; the part that has to
+// come from HBM as scattered rows moves at kHbmBytesPerPs.  A share h of the gathers is served
+// by the 256 MB memory-side cache: h = kMallShare * 256 MB / (bytes of B one pass touches),
+// at most 1, less the first touches (1 / uses per row of B).  The launch takes the longer of
+// the two, times a penalty when a window reads 256 bytes or less out of a wider row (the
+// partial rows use the fabric worse: x (1 + beta * log2(row bytes / g)^2)), plus a fixed cost.
+// Fitted on 150 measured shapes; the fastest predicted shape is within 3 % of the fastest
+// measured one on every matrix and feature size of the fit.
+constexpr double kHbmBytesPerPs = 5.528;
+constexpr double kMallShare = 0.5534;
+constexpr double kMallBytes = 256.0 * 1048576.0;
+constexpr double kBeta256 = 0.02, kBeta128 = 0.04, kSmallGather = 1.053;
+constexpr double kLaunchMs = 0.029;
+
+extern "C" int lf_model_spmm_ms(const int64_t* h_stats, int32_t num_parts, int32_t n_windows, int64_t num_rows,
+                                int64_t num_cols, int32_t feat_size, int32_t b_dtype, double* h_ms) {
+    LF_REQUIRE(h_stats && h_ms, LF_ERR_INVALID, "null argument");
+    LF_REQUIRE(num_parts >= 1 && n_windows >= 1 && num_rows >= 0 && num_cols >= 1, LF_ERR_INVALID, "bad shape");
+    LF_REQUIRE(feat_size >= 1 && feat_size % n_windows == 0, LF_ERR_INVALID,
+               "feat_size %d is not a multiple of %d windows", feat_size, n_windows);
+    LF_REQUIRE(b_dtype == LF_DTYPE_F32 || b_dtype == LF_DTYPE_BF16, LF_ERR_INVALID, "unknown B dtype %d", b_dtype);
+    const double elem = b_dtype == LF_DTYPE_BF16 ? 2.0 : 4.0;
+    const double n = (double)feat_size / n_windows;
+    const double g = n * elem, row_bytes = (double)feat_size * elem;
+    const double lg = std::log2(row_bytes / g);
+    const double beta = g < 256.0 ? kBeta128 : (g < 512.0 ? kBeta256 : 0.0);
+    const double penalty = (1.0 + beta * lg * lg) * (g < 256.0 ? kSmallGather : 1.0);
+    const double cols_p = (double)num_cols / num_parts;
+    double ms = 0.0;
+    for (int p = 0; p < num_parts; ++p) {
+        const int64_t* st = h_stats + (size_t)p * LF_MAX_CLASSES * LF_STATS_FIELDS;
+        double ell = 0, slots = 0, nnz = 0, touched = 0;
+        for (int k = 0; k < LF_MAX_CLASSES; ++k) {
+            const double cost_rows = (double)st[k * LF_STATS_FIELDS], distinct = (double)st[k * LF_STATS_FIELDS + 2];
+            const double e = k + 1 < LF_MAX_CLASSES ? distinct : std::max(cost_rows, distinct);
+            ell += e;
+            slots += e * (double)(1 << k);
+            nnz += (double)st[k * LF_STATS_FIELDS + 1];
+            touched += distinct;
+        }
+        const double slice = cols_p * g;
+        const double first = std::min(1.0, cols_p / std::max(nnz, 1.0));
+        const double h = std::min(1.0, kMallShare * kMallBytes / slice) * (1.0 - first);
+        const double gather = nnz * g;
+        const double other = (p == 0 ? (double)num_rows * n * 4.0 : touched * n * 8.0) + slots * 8.0 + ell * 8.0;
+        const double fabric_ps = (gather + other) * penalty / kFabricBytesPerPs;
+        const double hbm_ps = ((1.0 - h) * gather + other) * penalty / kHbmBytesPerPs;
+        ms += std::max(fabric_ps, hbm_ps) * 1e-9 + kLaunchMs;
+    }
+    *h_ms = ms * n_windows;
     return LF_OK;
 }

@@ -55,7 +55,7 @@ def _run_block_or_csr(g, fa, feat, fmt_name):
 def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="reference",
                    check_correctness=False, out_csv=None, keep_values=False, select_format=None):
     """Runs the flow for an iterable of MTX objects and returns a pandas DataFrame with the
-    reference's columns.  ``num_parts``: None = measure per (matrix, feature size); an int;
+    reference's columns.  ``num_parts``: None = from the launch-shape model per (matrix, feature size); an int;
     or a callable ``(g, feat_size) -> int``.  ``select_format``: None = CELL for every
     matrix; or a callable ``g -> "CELL" | "BSR" | "CSR"`` standing in for the reference's
     format-selection model (proc05.spmm.end-to-end.py:133)."""
@@ -88,7 +88,7 @@ def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="
         for feat in feat_sizes:
             t0 = time.perf_counter()
             if num_parts is None:
-                parts, windows = fa.choose_launch_shape(g, feat, cost_model=cost_model)
+                parts, windows = fa.predict_launch_shape(g, feat)
             elif callable(num_parts):
                 parts, windows = int(num_parts(g, feat)), 1
             else:

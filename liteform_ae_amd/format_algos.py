@@ -35,7 +35,8 @@ from .format_matrix_market import MTX, Bucket  # noqa: F401  (re-exported like t
 __all__ = ["build_hyb_format", "bench_hyb_with_config", "search_bucket_config",
            "CostModelSettings", "bench_bsrmm", "bench_naive", "spmm_bsr",
            "build_hyb_format_device", "HybFormat", "HybSpMM", "spmm_hyb", "spmm_csr",
-           "guess_num_partitions", "choose_num_partitions", "choose_launch_shape", "matrix_features_device"]
+           "guess_num_partitions", "choose_num_partitions", "choose_launch_shape", "matrix_features_device",
+           "predict_launch_shape", "model_spmm_ms", "row_overlap_device", "pick_launch_shape"]
 
 WIDTH_LIMIT = 1024   # format_algos.py:821
 
@@ -634,22 +635,77 @@ def matrix_features_device(g) -> dict:
     }
 
 
-MALL_BYTES = 256 << 20        # MI355X memory-side cache (Infinity Cache)
+ROW_OVERLAP_STRUCTURED = 0.3      # rows sharing this share of their columns with the row before: structured
+
+
+def row_overlap_device(g, max_samples: int = 8192) -> float:
+    """Share of a row's columns that also occur in the row before it, from a sample of rows
+    (lf_row_overlap).  Near 0 for graphs with scattered neighbours, 0.67 for a 27-point
+    stencil: one of the matrix features behind the launch-shape choice, next to
+    ``matrix_features_device``."""
+    torch = _torch()
+    lib = _lib.load()
+    dev = _device_csr(g)
+    out = np.zeros(2, dtype=np.int64)
+    scratch = torch.empty(2, dtype=torch.int64, device="cuda")
+    stride = max(1, dev.num_rows // max_samples)
+    _lib.check(lib.lf_row_overlap(_lib.ptr(dev.indptr), _lib.ptr(dev.indices), dev.num_rows, stride,
+                                  _lib.ptr(scratch), _lib.np_ptr(out, C.c_int64), _stream()))
+    return float(out[0]) / float(out[1]) if out[1] else 0.0
+
+
+def model_spmm_ms(stats, windows: int, num_rows: int, num_cols: int, feat_size: int, b_dtype: str = "f32") -> float:
+    """Predicted milliseconds of one product for the partitions described by ``stats``
+    (``bucket_statistics``) and ``windows`` feature windows (lf_model_spmm_ms; host only)."""
+    lib = _lib.load()
+    stats = np.ascontiguousarray(stats, dtype=np.int64)
+    out = C.c_double(0.0)
+    dt = {"f32": _lib.LF_DTYPE_F32, "bf16": _lib.LF_DTYPE_BF16}[b_dtype]
+    _lib.check(lib.lf_model_spmm_ms(_lib.np_ptr(stats, C.c_int64), int(stats.shape[0]), int(windows), int(num_rows),
+                                    int(num_cols), int(feat_size), dt, C.byref(out)))
+    return float(out.value)
+
+
+def pick_launch_shape(predicted: dict):
+    """The (partitions, windows) pair with the fewest launches among those predicted (or
+    measured) within 2 % of the fastest: fewer partitions mean less memory and fewer passes
+    over C, and differences below that are noise."""
+    fastest = min(predicted.values())
+    return min((k for k, t in predicted.items() if t <= 1.02 * fastest), key=lambda k: (k[0] * k[1], k[0]))
+
+
+def predict_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Sequence[int] = (1, 2, 3, 4),
+                         windows: Sequence[int] = None, return_predictions: bool = False):
+    """Column-partition count and feature-window count from a model of the MI355X memory
+    system, without composing a format or running a kernel.  Takes the place of the
+    reference's partition predictor, a RandomForest on eight matrix features
+    (proc05.spmm.end-to-end.py:82-97, 142) whose model file is not distributed.
+
+    Inputs: the bucket statistics of every candidate partition count (one pass over the row
+    pointer each, on the GPU) and the share of columns consecutive rows have in common.  A
+    structured matrix (stencil, band) reads B through the L2 whatever the shape: one
+    partition, one window.  Otherwise lf_model_spmm_ms prices every candidate and
+    ``pick_launch_shape`` takes the cheapest.  Costs well under a millisecond of GPU time where
+    ``choose_launch_shape`` spends hundreds composing and timing."""
+    if windows is None:
+        windows = _window_candidates(feat_size, b_dtype)
+    rows, cols = int(g.num_src_nodes()), int(g.num_dst_nodes())
+    predicted = {}
+    if row_overlap_device(g) >= ROW_OVERLAP_STRUCTURED:
+        best = (min(candidates), min(windows))
+    else:
+        for p in candidates:
+            stats, _ = bucket_statistics(g, p, with_columns=False)
+            for w in windows:
+                predicted[(p, w)] = model_spmm_ms(stats, w, rows, cols, feat_size, b_dtype)
+        best = pick_launch_shape(predicted)
+    return (best, predicted) if return_predictions else best
 
 
 def guess_num_partitions(g, feat_size: int, b_dtype: str = "f32") -> int:
-    """Column-partition count without measuring.  The reference predicts it with a trained
-    RandomForest (proc05.spmm.end-to-end.py:82-97) whose model file is not distributed; this
-    rule states what measurements on MI355X showed instead: partitions pay only when B is
-    several times larger than the 256 MB memory-side cache *and* B rows are reused often
-    (nnz / cols), because every extra partition re-reads and re-writes C once and adds one
-    ELL row per (row, partition) segment."""
-    elem = 2 if b_dtype == "bf16" else 4
-    b_bytes = g.num_dst_nodes() * feat_size * elem
-    reuse = g.num_edges() / max(1, g.num_dst_nodes())
-    if b_bytes <= 0.75 * MALL_BYTES or reuse < 8:
-        return 1
-    return int(min(4, max(1, round(b_bytes / (2.5 * MALL_BYTES)))))
+    """Column-partition count for a single pass over the features, from the model
+    (``predict_launch_shape`` with one window)."""
+    return predict_launch_shape(g, feat_size, b_dtype, windows=(1,))[0]
 
 
 def _window_candidates(feat_size: int, b_dtype: str) -> List[int]:
@@ -665,8 +721,8 @@ def choose_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Seq
     """Column-partition count and feature-window count by measurement: composes the format
     for every candidate partition count, times the fused kernel for every window count (a
     few runs each) and returns the pair (partitions, windows) with the fewest launches among
-    those within 2 % of the fastest.  Takes the place of the reference's partition predictor
-    (proc05.spmm.end-to-end.py:142); feature windows have no counterpart there."""
+    those within 2 % of the fastest.  The fallback (and the yardstick) of
+    ``predict_launch_shape``, which decides from a model in a fraction of the time."""
     torch = _torch()
     want = torch.float32 if b_dtype == "f32" else torch.bfloat16
     if windows is None:
@@ -690,10 +746,7 @@ def choose_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Seq
         del fmt
     if not timings:
         raise ValueError("no candidate partition count is usable for this matrix")
-    # fewest launches within 2 % of the fastest: fewer partitions mean less memory and fewer
-    # passes over C, and differences below that are run-to-run noise
-    fastest = min(timings.values())
-    best = min((k for k, t in timings.items() if t <= 1.02 * fastest), key=lambda k: (k[0] * k[1], k[0]))
+    best = pick_launch_shape(timings)
     return (best, timings) if return_timings else best
 
 

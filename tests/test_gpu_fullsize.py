@@ -164,3 +164,15 @@ def test_spmm_full_size_properties(big):
         assert (np.abs(got - ref) <= 1e-5 * bound).all()
         plan.close()
         del fmt, plan
+
+
+def test_launch_shape_model_on_the_headline_graph(big):
+    """The model's choice for the 2.45M-row graph: one pass at 64 features, two feature windows
+    at 128 (B is 1.25 GB against a 256 MB memory-side cache), as the measurements say."""
+    wl, fa, torch = big
+    g = wl.matrix
+    assert fa.row_overlap_device(g) < 0.01
+    assert fa.predict_launch_shape(g, 64) == (1, 1)
+    best, table = fa.predict_launch_shape(g, 128, return_predictions=True)
+    assert best == (1, 2)
+    assert 5.0 < table[best] < 8.0            # predicted milliseconds (measured: 6.2)

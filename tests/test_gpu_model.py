@@ -1,0 +1,86 @@
+"""The launch-shape model and the fold model against the GPU: the matrix features they read
+(lf_row_overlap) against numpy, the decisions on the benchmark shapes, and that a folded
+configuration the model asks for is not slower than the unfolded one."""
+import numpy as np
+import pytest
+
+from liteform_ae_amd.format_matrix_market import MTX
+
+from helpers import skewed_matrix
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def fa():
+    from liteform_ae_amd import format_algos
+    return format_algos
+
+
+def overlap_numpy(g, stride):
+    indptr, indices, _ = g.adj_tensors("csr")
+    both = seen = 0
+    for r in range(1, g.num_src_nodes(), stride):
+        a = indices[indptr[r - 1]:indptr[r]]
+        b = indices[indptr[r]:indptr[r + 1]]
+        both += len(np.intersect1d(a, b))
+        seen += len(b)
+    return both, seen
+
+
+def test_row_overlap_matches_numpy(fa):
+    import ctypes as C
+    import torch
+    from liteform_ae_amd import _lib
+    from liteform_ae_amd.synthetic import make_workload
+    lib = _lib.load()
+    rng = np.random.default_rng(61)
+    for g, stride in ((make_workload("cfg4", 0.01).matrix, 1), (make_workload("cfg4", 0.01).matrix, 7),
+                      (skewed_matrix(rng, 3000, 500, mean_deg=12, heavy_rows=2), 1),
+                      (MTX.from_coo(np.array([0]), np.array([0]), (1, 4)), 1)):
+        dev = fa._device_csr(g)
+        out = np.zeros(2, dtype=np.int64)
+        scratch = torch.empty(2, dtype=torch.int64, device="cuda")
+        _lib.check(lib.lf_row_overlap(dev.indptr.data_ptr(), dev.indices.data_ptr(), dev.num_rows, stride,
+                                      scratch.data_ptr(), _lib.np_ptr(out, C.c_int64), None))
+        assert tuple(out) == overlap_numpy(g, stride)
+    assert fa.row_overlap_device(make_workload("cfg4", 0.05).matrix) > 0.6      # 18 of 27 columns, less at the faces
+    assert fa.row_overlap_device(skewed_matrix(rng, 20000, 200000, mean_deg=10)) < 0.01
+
+
+def test_structured_and_small_matrices_get_one_launch(fa):
+    from liteform_ae_amd.synthetic import make_workload
+    best, table = fa.predict_launch_shape(make_workload("cfg4", 0.05).matrix, 256, return_predictions=True)
+    assert best == (1, 1) and table == {}                 # decided by the overlap of neighbouring rows
+    rng = np.random.default_rng(62)
+    g = skewed_matrix(rng, 30000, 30000, mean_deg=8, heavy_rows=2)
+    best, table = fa.predict_launch_shape(g, 128, return_predictions=True)
+    assert best == (1, 1) and set(table) == {(p, w) for p in (1, 2, 3, 4) for w in (1, 2)}
+    assert fa.guess_num_partitions(g, 128) == 1
+
+
+def test_a_folded_choice_is_not_slower(fa):
+    """33 entries per row: the MI355X fold model asks for 16-slot rows at N = 128; the product
+    with that configuration must not be slower than with the initial 64-slot rows."""
+    import torch
+    from liteform_ae_amd.synthetic import csr_from_row_degrees
+    rng = np.random.default_rng(33)
+    n = 1_000_000
+    indptr, indices = csr_from_row_degrees(np.full(n, 33), n, rng)
+    g = MTX.from_csr(indptr, indices, (n, n), data=rng.random(len(indices), dtype=np.float32))
+    feat = 128
+    cfg = fa.search_bucket_config(g, 1, fa.CostModelSettings(feat, 1, cost_model="gfx950"))
+    assert cfg == [[16]]
+    B = torch.rand((n, feat), device="cuda") - 0.5
+    C = torch.empty((n, feat), device="cuda")
+    times = {}
+    outs = {}
+    for name, widths in (("folded", cfg), ("initial", [[32, 64]])):    # a few rows lost a duplicate: 32 entries
+        fmt = fa.build_hyb_format_device(g, widths)
+        plan = fa.HybSpMM(fmt, feat)
+        times[name] = float(np.median(plan.time_ms(B, C, warmup=3, repeat=15)))
+        outs[name] = plan.run(B).clone()
+        plan.close()
+    assert times["folded"] <= 1.02 * times["initial"], times
+    # same product either way (a row's terms are added in the same order, in pieces of 16 or 64)
+    assert float((outs["folded"] - outs["initial"]).abs().max()) <= 1e-4
