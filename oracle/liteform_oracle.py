@@ -19,11 +19,15 @@ Two independent formulations are kept on purpose:
 Tests pin the sequential forms with hand-evaluated examples and brute force, and
 the closed forms against the sequential ones on random inputs.
 
-Pinning status: every function here is pinned by hand-worked known answers,
-invariants or brute force in tests/test_oracle_*.py.  The reference holds no
-golden vectors for this path and its GPU kernel comes from an external code
-generator, so the SpMM result is anchored on scipy CSR(f64) @ dense(f64), the
-reference's own CPU product (FM:89-99).
+Pinning status: every function of the format path (initial buckets, single-row
+fix-up, cost function, fold search, hyb builder) is pinned twice: by hand-worked
+known answers, invariants and brute force (tests/test_oracle_format.py,
+tests/test_golden_examples.py), and bit for bit - float costs included - against
+vectors produced by the reference's own functions on 21 seeded matrices
+(tests/golden/search_vectors.*, tests/test_reference_vectors.py).  The reference's
+GPU kernel comes from an external code generator and has no recorded outputs, so
+the SpMM result is anchored on scipy CSR(f64) @ dense(f64), the reference's own
+CPU product (FM:89-99).
 """
 from __future__ import annotations
 
