@@ -35,6 +35,8 @@ constexpr int kTileRows = 512;      // ELL rows per tile at most (<= tile_slots)
 #endif
 constexpr int kCoopSlots = LF_COOP_SLOTS;    // a source row with more slab slots is reduced by a whole workgroup
 constexpr int kChunkSlots = LF_CHUNK_SLOTS;  // ... in chunks of this many slots (a whole number of ELL rows)
+constexpr int kChunkSlotsLarge = 8192;       // ... or this many, in a matrix of at least kLargeMatrixSlots slots
+constexpr long long kLargeMatrixSlots = 4ll << 20;
 constexpr int kXcds = 8;
 constexpr int kPartBytesMax = 16384;   // LDS for per-ELL-row sums of a balanced segment tile at most
 constexpr int kUnroll = LF_UNROLL;  // B-row gathers in flight per sub-wave
