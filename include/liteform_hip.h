@@ -250,10 +250,13 @@ int lf_spmm_destroy(lf_spmm_plan* plan);
  * format_algos.py:491-520). */
 int lf_spmm_set_windows(lf_spmm_plan* plan, int32_t n_windows);
 
-/* h_info[0..7] = tiles, workgroups per launch, launches per run, LDS bytes per workgroup,
- * heavy (split) segments, partial rows, rows cleared by partition 0, buckets served four rows
- * at a time with shared gathers (consecutive rows holding mostly the same columns; the
- * environment variable LF_ROW_GROUPS=0 at plan creation turns that path off). */
+/* h_info[0..LF_SPMM_INFO_FIELDS-1] = tiles, workgroups per launch, launches per run, LDS bytes
+ * per workgroup, heavy (split) segments, partial rows, rows cleared by partition 0, buckets
+ * served with shared gathers (rows close together holding mostly the same columns), and how
+ * many of those are served as 16-row cells on the matrix cores rather than four consecutive
+ * rows at a time.  The environment variable LF_ROW_GROUPS at plan creation: 0 turns both
+ * paths off, 4 keeps the four-row groups only. */
+#define LF_SPMM_INFO_FIELDS 9
 int lf_spmm_info(const lf_spmm_plan* plan, int64_t* h_info);
 
 /* Timing helper, the counterpart of the reference's profile_tvm_ms / run_100_times

@@ -21,6 +21,7 @@ LF_ERR_WORKSPACE = -6
 
 LF_MAX_CLASSES = 11
 LF_STATS_FIELDS = 4
+LF_SPMM_INFO_FIELDS = 9
 LF_DTYPE_F32 = 0
 LF_DTYPE_BF16 = 1
 LF_COST_REFERENCE = 0

@@ -1065,7 +1065,7 @@ struct lf_spmm_plan {
     Group* d_groups = nullptr;
     HeavyRow* d_heavy = nullptr;
     float* d_partials = nullptr;
-    int64_t info[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int64_t info[LF_SPMM_INFO_FIELDS] = {0};
 };
 
 namespace {
@@ -1635,6 +1635,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     plan->info[6] = n_zero;
     (void)occ;
     plan->info[7] = (int64_t)(merged.size() + cells.size());
+    plan->info[8] = (int64_t)cells.size();
     LF_TRY_HIP(hipStreamSynchronize(s));     // the tables are complete: the plan may run on any stream
     if (free_temporaries(plan) != LF_OK) return bail(lf::fail(LF_ERR_HIP, "hipFree failed on plan-time scratch"));
     *out_plan = plan;

@@ -105,7 +105,7 @@ def test_raw_abi_end_to_end(env):
             k += 1
     plan = C.c_void_p()
     assert lib.lf_spmm_create(C.byref(plan), descs, nb, P, rows, cols, feat, 0, None) == 0
-    info = np.zeros(8, np.int64)
+    info = np.zeros(L.LF_SPMM_INFO_FIELDS, np.int64)
     assert lib.lf_spmm_info(plan, L.np_ptr(info, C.c_int64)) == 0 and info[2] == P and info[0] > 0
     B = rng.uniform(-1, 1, size=(cols, feat)).astype(np.float32)
     dB = dev(torch, B, np.float32)

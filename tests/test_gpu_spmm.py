@@ -31,7 +31,7 @@ def to_bf16_exact(torch, B):
     return torch.from_numpy(B).to(torch.bfloat16)
 
 
-def check(fa, torch, g, widths, feat, b_dtype="f32", seed=0):
+def check(fa, torch, g, widths, feat, b_dtype="f32", seed=0, windows=1):
     rng = np.random.default_rng(seed)
     nr, nc = g.coo_mtx.shape
     B = rng.uniform(-1, 1, size=(nc, feat)).astype(np.float32)
@@ -42,7 +42,7 @@ def check(fa, torch, g, widths, feat, b_dtype="f32", seed=0):
     else:
         Bd = torch.from_numpy(B).cuda()
     fmt = fa.build_hyb_format_device(g, widths)
-    plan = fa.HybSpMM(fmt, feat, b_dtype)
+    plan = fa.HybSpMM(fmt, feat, b_dtype, windows=windows)
     C1 = plan.run(Bd).cpu().numpy()
     C2 = plan.run(Bd).cpu().numpy()
     plan.close()
@@ -320,6 +320,50 @@ def mixed_band_matrix(rng, n):
         cols.append(np.arange(lo, hi))
     rows, cols = np.concatenate(rows), np.concatenate(cols)
     return MTX.from_coo(rows, cols, (n, n), data=rng.uniform(-1, 1, size=len(rows)).astype(np.float32))
+
+
+def grid_stencil(rng, dims, reach=1):
+    """Every point of a grid (first dimension fastest) coupled to its neighbours within `reach`
+    in every direction: 9 columns per interior row in two dimensions, 27 in three."""
+    shape = tuple(reversed(dims))
+    idx = np.arange(int(np.prod(dims))).reshape(shape)
+    rows, cols = [], []
+    offsets = np.stack(np.meshgrid(*[np.arange(-reach, reach + 1)] * len(dims), indexing="ij"), -1).reshape(-1, len(dims))
+    for off in offsets:
+        src = tuple(slice(max(0, -o), s - max(0, o)) for o, s in zip(off, shape))
+        dst = tuple(slice(max(0, o), s - max(0, -o)) for o, s in zip(off, shape))
+        rows.append(idx[src].ravel())
+        cols.append(idx[dst].ravel())
+    rows, cols = np.concatenate(rows), np.concatenate(cols)
+    n = idx.size
+    return MTX.from_coo(rows, cols, (n, n), data=rng.uniform(-1, 1, size=len(rows)).astype(np.float32))
+
+
+@pytest.mark.parametrize("feat,windows", [(256, 1), (512, 2)])
+def test_grid_stencils_are_served_as_cells(fa, torch, feat, windows, monkeypatch):
+    """fp32 B, 256 features per pass: buckets of a stencil become 16-row cells (neighbours in
+    every direction of the grid, found from the column differences) on the matrix cores; the
+    product is the plain path's to rounding and within the bound of the float64 oracle."""
+    rng = np.random.default_rng(77 + feat)
+    for g, widths in ((grid_stencil(rng, (37, 29, 23)), [[8, 16, 32]]),        # 27 points, ragged cell edges
+                      (grid_stencil(rng, (150, 131)), [[4, 8, 16]]),           # 9 points, two strides
+                      (grid_stencil(rng, (64, 40, 16)), [[32]]),               # one bucket for faces and interior
+                      (banded_matrix(rng, 9001, 10), [[8, 16, 32]])):          # one stride
+        C1, info = check(fa, torch, g, widths, feat, "f32", seed=feat, windows=windows)
+        assert info["cell_buckets"] >= 1, (widths, info)
+        monkeypatch.setenv("LF_ROW_GROUPS", "4")
+        C4, info4 = check(fa, torch, g, widths, feat, "f32", seed=feat, windows=windows)
+        monkeypatch.setenv("LF_ROW_GROUPS", "0")
+        C0, info0 = check(fa, torch, g, widths, feat, "f32", seed=feat, windows=windows)
+        monkeypatch.delenv("LF_ROW_GROUPS")
+        assert info4["cell_buckets"] == 0 and info4["row_group_buckets"] >= 1
+        assert info0["row_group_buckets"] == 0
+        # same terms per row in ascending column order on all three paths: they differ only in
+        # the rounding of fused multiply-adds (|a|, |b| < 1, at most 27 terms)
+        assert np.abs(C1 - C0).max() <= 2e-5 and np.abs(C4 - C0).max() <= 2e-5
+    g = skewed_matrix(rng, 20000, 30000, mean_deg=20, heavy_rows=0)
+    _, info = check(fa, torch, g, [[8, 16, 32, 64]], feat, "f32", seed=feat, windows=windows)
+    assert info["cell_buckets"] == 0
 
 
 @pytest.mark.parametrize("feat,b_dtype", [(32, "f32"), (64, "f32"), (128, "f32"), (256, "f32"), (256, "bf16"),
