@@ -228,7 +228,6 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 // addresses then go through the scalar cache and are counted apart from the vector loads
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef const i32x4 __attribute__((address_space(4)))* ConstInt4Ptr;
 typedef const f32x4 __attribute__((address_space(1)))* GlobalFloat4Ptr;
 typedef const i32x4 __attribute__((address_space(1)))* GlobalInt4Ptr;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -253,7 +252,23 @@ template <> __device__ __forceinline__ void unpack_features<bf16_t>(const u32x4&
 // the entry's 16 weights (lane l supplies the weight of row l % 16) and the c-th feature of
 // every lane, and adds the four 16 x 16 outer products to accumulator c.  In accumulator c,
 // register g of lane l belongs to row 4*(l/16) + g%4 and feature VEC*(16*(g/4) + l%16) + c.
-// Entries are walked in half-batches of four: while one is added, the other's loads are in flight.
+//
+// Columns and weights of a cell are read once and are never in a cache, so every load of them
+// waits out the full memory latency.  Fetched piecemeal next to the gathers they steer (four
+// columns and one weight vector per half-batch) that latency was paid 24 times per cell, one
+// after the other: 100^3 stencil at N = 256, 0.75 ms, and still 0.73 ms with every gather
+// turned into a cache hit.  Here the whole cell's columns arrive with one load (lane l: entries
+// 4l .. 4l+3; a cell has at most 256) and its weights with up to eight full-width loads that
+// go to LDS; the loop takes columns out of registers (readlane) and weights out of LDS and
+// only ever waits for gathers: 0.67 ms.  Entries are walked in half-batches of four with three
+// in flight (0.645 ms; two 0.67, four 0.65, six 0.66).  C is stored past the caches' retention
+// (non-temporal: 0.765 -> 0.75 ms before the other changes), which leaves more of the L2 to B.
+// Measured on the way: weights straight into LDS with global_load_lds (no staging registers,
+// three wavefronts per SIMD instead of two) 0.75-0.85 ms; three or four wavefronts per SIMD by
+// register limit 0.68 / 0.77 ms.
+constexpr int kCellChunk = 128;            // merged entries whose weights a wavefront holds in LDS at a time
+constexpr int kCellDepth = 3;              // half-batches of gathers in flight
+
 template <typename BT>
 __global__ void __launch_bounds__(kWG)
 spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const void* __restrict__ B,
@@ -261,6 +276,9 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
     constexpr int VEC = Dense<BT>::kVec;
     constexpr int G = kCellRows;
     constexpr int H = 4;
+    constexpr int D = kCellDepth;
+    constexpr int kLoads = kCellChunk * 4 / 64;       // full-width loads that bring a chunk's weights
+    __shared__ f32x4 s_w[kCellTileCells][kCellChunk * 4];
     const int xcd = blockIdx.x % kXcds;
     long long v = blockIdx.x / kXcds;
     for (int bi = 0; bi < n_buckets; ++bi) {
@@ -278,7 +296,7 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
         int my_off = 0;
         if (first + lane <= b.n_cells) my_off = b.eoff[first + lane];
         else my_off = b.eoff[b.n_cells];
-        const Lane<64, 1, VEC> ln(lane, feat, ldb, ldc);
+        f32x4* sw = s_w[wave];
         for (int step = 0; step < kCellsPerWave; ++step) {
         const int slot = step * kCellTileCells + wave;
         const long long cell = first + slot;
@@ -286,11 +304,10 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
         const int e0 = __builtin_amdgcn_readlane(my_off, slot);
         const int m = __builtin_amdgcn_readlane(my_off, slot + 1) - e0;           // a multiple of kCellBatch
         if (m == 0) continue;
-        const int32_t* __restrict__ ecol = b.ecol + e0;
         // (pointers read out of the bucket record are generic to the compiler; saying that they
         // are global memory keeps their loads off the LDS counter)
-        const GlobalFloat4Ptr wq = reinterpret_cast<GlobalFloat4Ptr>(reinterpret_cast<uintptr_t>(b.wq)) +
-                                   ((size_t)e0 / 4 * G + (lane & 15));
+        const int cidx = min(4 * lane, m - 4);
+        const i32x4 colv = *reinterpret_cast<GlobalInt4Ptr>(reinterpret_cast<uintptr_t>(b.ecol + e0 + cidx));
         floatx16 acc[VEC];
 #pragma unroll
         for (int c = 0; c < VEC; ++c)
@@ -301,47 +318,65 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
         const char* b_bytes = reinterpret_cast<const char*>(B);
         const size_t row_bytes = (size_t)ldb * sizeof(BT);
         const uint32_t lane_off = (uint32_t)lane * 16u;
-        auto issue = [&](int j, f32x4& w, u32x4 (&x)[H]) {
-            // (no branch around the loads: the compiler counts outstanding loads per path)
-            const int jj = j < m ? j : m - H;                 // past the end: the last half-batch again, unused
-            // the columns come through the scalar cache (wavefront-uniform addresses): a vector
-            // load here would have to be waited for in order, behind the gathers still in flight
-            const i32x4 cols4 = *reinterpret_cast<ConstInt4Ptr>(reinterpret_cast<uintptr_t>(ecol + jj));
-            const int c[H] = {cols4.x, cols4.y, cols4.z, cols4.w};
-            w = wq[(size_t)(jj >> 2) * G];
+        for (int base = 0; base < m; base += kCellChunk) {
+            const int mc = min(kCellChunk, m - base);
+            // the chunk's weights, [mc / 4][16 rows] float4, are contiguous: lane l takes float4 l of every 64
+            const GlobalFloat4Ptr wsrc = reinterpret_cast<GlobalFloat4Ptr>(reinterpret_cast<uintptr_t>(b.wq)) +
+                                         (size_t)(e0 + base) * 4;
+            f32x4 wreg[kLoads];
 #pragma unroll
-            for (int u = 0; u < H; ++u) {
-                const char* row = b_bytes + (size_t)(uint32_t)c[u] * row_bytes;
-                x[u] = *reinterpret_cast<GlobalU32x4Ptr>(reinterpret_cast<uintptr_t>(row + lane_off));
+            for (int i = 0; i < kLoads; ++i)
+                if (i * 64 < mc * 4) wreg[i] = __builtin_nontemporal_load(wsrc + min(i * 64 + lane, mc * 4 - 1));
+            auto issue = [&](int j, f32x4& w, u32x4 (&x)[H], bool with_w) {
+                // (no branch around the loads: the compiler counts outstanding loads per path)
+                const int jj = j < mc ? j : mc - H;               // past the end: the last half-batch again, unused
+                const int q = (base + jj) >> 2;
+                const int c[H] = {__builtin_amdgcn_readlane(colv.x, q), __builtin_amdgcn_readlane(colv.y, q),
+                                  __builtin_amdgcn_readlane(colv.z, q), __builtin_amdgcn_readlane(colv.w, q)};
+                if (with_w) w = sw[(jj >> 2) * G + (lane & 15)];
+#pragma unroll
+                for (int u = 0; u < H; ++u) {
+                    const char* row = b_bytes + (size_t)(uint32_t)c[u] * row_bytes;
+                    x[u] = *reinterpret_cast<GlobalU32x4Ptr>(reinterpret_cast<uintptr_t>(row + lane_off));
+                }
+            };
+            auto add_rows = [&](const f32x4& w, const u32x4 (&x)[H]) {
+                const float wu[H] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                for (int u = 0; u < H; ++u) {
+                    float f[VEC];
+                    unpack_features<BT>(x[u], f);
+#pragma unroll
+                    for (int c = 0; c < VEC; ++c)
+                        acc[c] = __builtin_amdgcn_mfma_f32_16x16x1f32(wu[u], f[c], acc[c], 0, 0, 0);
+                }
+            };
+            // The scheduling fences keep each group of loads ahead of the arithmetic of the
+            // half-batches before it; left alone, the compiler sinks the loads to just before
+            // their first use and every half-batch waits out the full memory latency.
+            f32x4 wr[D];
+            u32x4 xr[D][H];
+            issue(0, wr[0], xr[0], false);                        // the first gathers leave before the weights are in
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i)
+                if (i * 64 < mc * 4) sw[i * 64 + lane] = wreg[i];
+            // one wavefront writes and reads this part of LDS, and LDS operations of a wavefront
+            // complete in order: no barrier between the workgroup's wavefronts is needed
+            __builtin_amdgcn_wave_barrier();
+            wr[0] = sw[lane & 15];
+#pragma unroll
+            for (int k = 1; k < D - 1; ++k) issue(k * H, wr[k], xr[k], true);
+            for (int j = 0; j < mc; j += D * H) {
+#pragma unroll
+                for (int k = 0; k < D; ++k) {
+                    issue(j + (D - 1 + k) * H, wr[(D - 1 + k) % D], xr[(D - 1 + k) % D], true);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (k == 0 || j + k * H < mc) add_rows(wr[k], xr[k]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
-        };
-        auto add_rows = [&](const f32x4& w, const u32x4 (&x)[H]) {
-            const float wu[H] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-            for (int u = 0; u < H; ++u) {
-                float f[VEC];
-                unpack_features<BT>(x[u], f);
-#pragma unroll
-                for (int c = 0; c < VEC; ++c)
-                    acc[c] = __builtin_amdgcn_mfma_f32_16x16x1f32(wu[u], f[c], acc[c], 0, 0, 0);
-            }
-        };
-        // Two half-batches are in flight at a time (a third measured slower: 0.80 against
-        // 0.76 ms).  The scheduling fences keep each group of loads ahead of the arithmetic of
-        // the other half-batch; left alone, the compiler sinks the loads to just before their
-        // first use and every half-batch waits out the full memory latency.
-        f32x4 wa, wb;
-        u32x4 xa[H], xb[H];
-        issue(0, wa, xa);
-        for (int j = 0; j < m; j += 2 * H) {
-            issue(j + H, wb, xb);
-            __builtin_amdgcn_sched_barrier(0);
-            add_rows(wa, xa);
-            __builtin_amdgcn_sched_barrier(0);
-            issue(j + 2 * H, wa, xa);
-            __builtin_amdgcn_sched_barrier(0);
-            add_rows(wb, xb);
-            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_wave_barrier();
         }
         // rows of this lane's registers: 4*(lane/16) .. +3
         const i32x4 my_rows = *reinterpret_cast<GlobalInt4Ptr>(reinterpret_cast<uintptr_t>(b.rows + cell * G + 4 * (lane >> 4)));
@@ -353,12 +388,9 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
             float* dst = C + (size_t)row * ldc + VEC * (16 * (g >> 2) + (lane & 15));
 #pragma unroll
             for (int i = 0; i < VEC; i += 4) {
-                float4 o = make_float4(acc[i][g], acc[i + 1][g], acc[i + 2][g], acc[i + 3][g]);
-                if (accumulate) {
-                    const float4 old = *reinterpret_cast<const float4*>(dst + i);
-                    o.x += old.x; o.y += old.y; o.z += old.z; o.w += old.w;
-                }
-                *reinterpret_cast<float4*>(dst + i) = o;
+                f32x4 o = {acc[i][g], acc[i + 1][g], acc[i + 2][g], acc[i + 3][g]};
+                if (accumulate) o += *reinterpret_cast<const f32x4*>(dst + i);
+                __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(dst + i));
             }
         }
         }
