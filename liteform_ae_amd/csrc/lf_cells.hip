@@ -40,7 +40,8 @@ namespace {
 
 constexpr int kCellRows = 16;              // rows of a cell: the row dimension of the outer-product instruction
 constexpr int kCellBatch = 8;              // merged entries are padded to whole batches of this many
-constexpr int kCellTileCells = 4;          // cells a workgroup is on at a time: one per wavefront
+constexpr int kCellTileCells = 4;          // cells a workgroup is on at a time: one per wavefront (one or two
+                                           // per workgroup measured 2 % slower)
 #ifndef LF_CELLS_PER_WAVE
 #define LF_CELLS_PER_WAVE 1
 #endif
@@ -270,7 +271,7 @@ constexpr int kCellChunk = 128;            // merged entries whose weights a wav
 constexpr int kCellDepth = 3;              // half-batches of gathers in flight
 
 template <typename BT>
-__global__ void __launch_bounds__(kWG)
+__global__ void __launch_bounds__(64 * kCellTileCells)
 spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const void* __restrict__ B,
                  float* __restrict__ C, int feat, int ldb, int ldc, int accumulate) {
     constexpr int VEC = Dense<BT>::kVec;
@@ -577,7 +578,7 @@ int cells_launch(const LfCellBucket* d_buckets, int n_buckets, int grid, int b_d
                  int feat, int ldb, int ldc, int accumulate, hipStream_t s) {
     if (n_buckets <= 0 || grid <= 0) return LF_OK;
     LF_REQUIRE(b_dtype == LF_DTYPE_F32, LF_ERR_UNSUPPORTED, "cells are built for fp32 operands only");
-    spmm_cell_kernel<float><<<grid, kWG, 0, s>>>(d_buckets, n_buckets, B, C, feat, ldb, ldc, accumulate);
+    spmm_cell_kernel<float><<<grid, 64 * kCellTileCells, 0, s>>>(d_buckets, n_buckets, B, C, feat, ldb, ldc, accumulate);
     LF_HIP(hipGetLastError());
     return LF_OK;
 }
