@@ -153,7 +153,8 @@ int lf_model_spmm_ms(const int64_t* h_stats, int32_t num_parts, int32_t n_window
                      int64_t num_cols, int32_t feat_size, int32_t b_dtype, double* h_ms);
 
 /* Share of the entries of every sample_stride-th row whose column also occurs in the row
- * before it: h_out = {entries in both rows, entries looked at}.  Near 0 for matrices with
+ * before it (the first 64 entries of either row): h_out = {entries in both rows, entries
+ * looked at}.  Near 0 for matrices with
  * scattered columns, 0.67 for a 27-point stencil; rows that share columns read B through the
  * L2 and gain nothing from column partitions or feature windows.  d_scratch: 16 bytes of
  * device memory.  Synchronises the stream.  (One of the inputs of the launch-shape choice, as

@@ -149,7 +149,11 @@ row_features_kernel(const int32_t* __restrict__ indptr, int64_t rows, unsigned l
 }
 
 // out[0] += entries of row r that also occur in row r - 1, out[1] += entries of row r, for every
-// stride-th row r >= 1 (two-pointer walk over the two ascending column lists)
+// stride-th row r >= 1 (two-pointer walk over the two ascending column lists).  Only the first
+// kOverlapEntries entries of either row are looked at: one thread walks a pair of rows, and a
+// sample that lands on a row of 100,000 entries would otherwise take longer than composing the
+// whole format (11 ms against 0.3 ms for a 500k x 2M matrix with 50 such rows).
+constexpr int kOverlapEntries = 64;
 __global__ void __launch_bounds__(kBlock)
 row_overlap_kernel(const int32_t* __restrict__ indptr, const int32_t* __restrict__ indices, int64_t rows,
                    int64_t stride, unsigned long long* __restrict__ out) {
@@ -158,7 +162,7 @@ row_overlap_kernel(const int32_t* __restrict__ indptr, const int32_t* __restrict
         const int64_t r = 1 + i * stride;
         if (r >= rows) break;
         int a = indptr[r - 1], b = indptr[r];
-        const int a_end = b, b_end = indptr[r + 1];
+        const int a_end = min(b, a + kOverlapEntries), b_end = min(indptr[r + 1], b + kOverlapEntries);
         seen += (unsigned long long)(b_end - b);
         while (a < a_end && b < b_end) {
             const int ca = indices[a], cb = indices[b];
