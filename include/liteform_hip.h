@@ -214,11 +214,18 @@ int lf_hyb_build(const int32_t* d_indptr, const int32_t* d_indices, const float*
  * (format_algos.py:552-578: values float32, rows int32, cols int32 row-major), plus the
  * optional meta array of lf_hyb_build (NULL: derived from rows/vals at create time).
  * The slabs must stay alive and unchanged while the plan exists.
- * At creation, buckets of 8..64-slot rows whose consecutive rows hold mostly the same columns
- * (stencils, banded and block-structured matrices) are rewritten inside the plan as groups
- * of four rows with merged column lists, so that one read of a B row serves up to four
- * output rows; this costs plan time and memory (about 21 bytes per merged entry) only
- * where a sample of the bucket shows at least 30 % fewer reads.
+ * At creation every slab is checked on the GPU: a column outside [0, num_cols), a row outside
+ * [0, num_rows) or a meta word that does not fit its bucket gives LF_ERR_INVALID, a source row
+ * spanning more ELL rows than a meta word can count LF_ERR_UNSUPPORTED (the reference casts the
+ * arrays it is given and launches, format_algos.py:568-577).
+ * At creation, buckets of 8..64-slot rows whose neighbouring rows hold mostly the same columns
+ * (stencils, banded and block-structured matrices) are rewritten inside the plan so that one
+ * read of a B row serves several output rows: as groups of four consecutive rows with merged
+ * column lists (about 21 bytes per merged entry), or - float32 B, 256 features per pass - as
+ * cells of 16 rows that are neighbours in up to three directions of the underlying grid (the
+ * directions are read off the column differences of sampled rows; 68 bytes per merged entry),
+ * accumulated with the fp32 outer-product matrix instruction.  This costs plan time and memory
+ * only where a sample of the bucket shows at least 30 % fewer reads.
  * feat_size must be a multiple of 32 (float32 B) or 64 (bf16 B), at most 1024.
  * ------------------------------------------------------------------------------------ */
 typedef struct lf_bucket_desc {

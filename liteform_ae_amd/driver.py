@@ -116,8 +116,8 @@ def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="
                                                     num_col_parts=parts, use_implicit_unroll=True,
                                                     check_correctness=check_correctness,
                                                     feature_windows=windows)
-                print(f"name: {g.name} format: {fmt_name} feat_size: {feat} num_partitions: {parts} "
-                      f"cost_model_config: {cfg} bucket_config: {bucket_config} exe_time: {exe_time}", flush=True)
+                print(f"[{g.name}] {fmt_name} N={feat} partitions={parts} windows={windows} widths={bucket_config} "
+                      f"search={time_bucket * 1e3:.3f} ms compose={compose_ms:.3f} ms kernel={exe_time:.4f} ms", flush=True)
             except Exception as e:                                     # proc05:178-180
                 exe_time = math.inf
                 print(e, file=sys.stderr)
