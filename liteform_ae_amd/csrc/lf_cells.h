@@ -34,8 +34,8 @@ constexpr int kCellEntriesCap = 256;   // merged entries of one cell at most
 int cells_build(const lf_bucket_desc& b, const int32_t* d_meta, int64_t num_rows, int64_t row_bytes, hipStream_t s,
                 std::vector<void*>* owned, std::vector<void*>* temp, LfCellBucket* out, bool* accepted);
 
-// One launch over `n_buckets` rewritten buckets (d_buckets: device array).  fp32 B with 256
-// features: one 16-byte load per lane of a 64-lane wavefront covers a row of B.
+// One launch over `n_buckets` rewritten buckets (d_buckets: device array).  fp32 B with 128 or
+// 256 features per pass: one 16-byte load per lane, 32 or 64 lanes per row of B.
 int cells_launch(const LfCellBucket* d_buckets, int n_buckets, int grid, int b_dtype, const void* B, float* C,
                  int feat, int ldb, int ldc, int accumulate, hipStream_t s);
 

@@ -270,13 +270,28 @@ template <> __device__ __forceinline__ void unpack_features<bf16_t>(const u32x4&
 constexpr int kCellChunk = 128;            // merged entries whose weights a wavefront holds in LDS at a time
 constexpr int kCellDepth = 3;              // half-batches of gathers in flight
 
-template <typename BT>
+//
+// LPR lanes cover a row of B (64: 256 fp32 or 512 bf16 features per pass; 32 and 16: half and a
+// quarter of that).  With LPR < 64 one gather instruction fetches the rows of E = 64 / LPR
+// consecutive merged entries, one per group of LPR lanes, and the instruction's four blocks
+// fall to different entries: block b belongs to entry b / (4 / E) and feature block b % (4 / E).
+// A lane then holds E partial sums of every output element (entries e, e + E, e + 2E, ...,
+// each in ascending column order), which it adds in the order e = 0 .. E-1 before the store.
+// 27-point stencil on 100^3, cells against four-row groups: fp32 N = 256 0.66 / 1.12 ms,
+// N = 128 0.40 / 0.52 ms, N = 64 0.29 / 0.30 ms (a tie: not worth the rewrite, so 16 lanes per
+// row are not launched); bf16 B doubles the matrix instructions per gathered byte and leaves
+// one wavefront per SIMD (128 accumulator registers): N = 512 / 256 / 128 1.87 / 1.15 / 0.68 ms
+// against 1.51 / 0.72 / 0.41 ms, so bf16 operands stay with the row groups.
+template <typename BT, int LPR>
 __global__ void __launch_bounds__(64 * kCellTileCells)
 spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const void* __restrict__ B,
                  float* __restrict__ C, int feat, int ldb, int ldc, int accumulate) {
     constexpr int VEC = Dense<BT>::kVec;
     constexpr int G = kCellRows;
-    constexpr int H = 4;
+    constexpr int E = 64 / LPR;                       // merged entries per gather instruction
+    constexpr int H = E == 4 ? 2 : 4;                 // gather instructions per half-batch
+    constexpr int HE = H * E;                         // merged entries per half-batch: 4 or 8
+    constexpr int NB = 4 / E;                         // feature blocks of 16 lanes per row of B
     constexpr int D = kCellDepth;
     constexpr int kLoads = kCellChunk * 4 / 64;       // full-width loads that bring a chunk's weights
     __shared__ f32x4 s_w[kCellTileCells][kCellChunk * 4];
@@ -328,34 +343,56 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
 #pragma unroll
             for (int i = 0; i < kLoads; ++i)
                 if (i * 64 < mc * 4) wreg[i] = __builtin_nontemporal_load(wsrc + min(i * 64 + lane, mc * 4 - 1));
-            auto issue = [&](int j, f32x4& w, u32x4 (&x)[H], bool with_w) {
+            const int sub = lane / LPR;                           // which of the E entries of an instruction this lane gathers
+            const uint32_t sub_off = (uint32_t)(lane % LPR) * 16u;
+            auto issue = [&](int j, f32x4 (&w)[(HE + 3) / 4], u32x4 (&x)[H], bool with_w) {
                 // (no branch around the loads: the compiler counts outstanding loads per path)
-                const int jj = j < mc ? j : mc - H;               // past the end: the last half-batch again, unused
-                const int q = (base + jj) >> 2;
-                const int c[H] = {__builtin_amdgcn_readlane(colv.x, q), __builtin_amdgcn_readlane(colv.y, q),
-                                  __builtin_amdgcn_readlane(colv.z, q), __builtin_amdgcn_readlane(colv.w, q)};
-                if (with_w) w = sw[(jj >> 2) * G + (lane & 15)];
+                const int jj = j < mc ? j : mc - HE;              // past the end: the last half-batch again, unused
+                const int q = (base + jj) >> 2;                   // jj is a multiple of 4: entry n sits in lane n / 4, component n % 4
+                int c[HE];
+#pragma unroll
+                for (int t = 0; t < HE; t += 4) {
+                    c[t] = __builtin_amdgcn_readlane(colv.x, q + t / 4);
+                    c[t + 1] = __builtin_amdgcn_readlane(colv.y, q + t / 4);
+                    c[t + 2] = __builtin_amdgcn_readlane(colv.z, q + t / 4);
+                    c[t + 3] = __builtin_amdgcn_readlane(colv.w, q + t / 4);
+                }
+                if (with_w) {
+#pragma unroll
+                    for (int t = 0; t < (HE + 3) / 4; ++t) w[t] = sw[((jj >> 2) + t) * G + (lane & 15)];
+                }
 #pragma unroll
                 for (int u = 0; u < H; ++u) {
-                    const char* row = b_bytes + (size_t)(uint32_t)c[u] * row_bytes;
-                    x[u] = *reinterpret_cast<GlobalU32x4Ptr>(reinterpret_cast<uintptr_t>(row + lane_off));
+                    if constexpr (E == 1) {
+                        const char* row = b_bytes + (size_t)(uint32_t)c[u] * row_bytes;
+                        x[u] = *reinterpret_cast<GlobalU32x4Ptr>(reinterpret_cast<uintptr_t>(row + lane_off));
+                    } else {
+                        int col = c[u * E];
+#pragma unroll
+                        for (int e = 1; e < E; ++e) col = sub == e ? c[u * E + e] : col;
+                        const char* row = b_bytes + (size_t)(uint32_t)col * row_bytes;
+                        x[u] = *reinterpret_cast<GlobalU32x4Ptr>(reinterpret_cast<uintptr_t>(row + sub_off));
+                    }
                 }
             };
-            auto add_rows = [&](const f32x4& w, const u32x4 (&x)[H]) {
-                const float wu[H] = {w.x, w.y, w.z, w.w};
+            auto add_rows = [&](const f32x4 (&w)[(HE + 3) / 4], const u32x4 (&x)[H]) {
 #pragma unroll
                 for (int u = 0; u < H; ++u) {
+                    // the weight of this lane's row at the entry this lane's block belongs to
+                    float wu = w[(u * E) / 4][(u * E) % 4];
+#pragma unroll
+                    for (int e = 1; e < E; ++e) wu = sub == e ? w[(u * E + e) / 4][(u * E + e) % 4] : wu;
                     float f[VEC];
                     unpack_features<BT>(x[u], f);
 #pragma unroll
                     for (int c = 0; c < VEC; ++c)
-                        acc[c] = __builtin_amdgcn_mfma_f32_16x16x1f32(wu[u], f[c], acc[c], 0, 0, 0);
+                        acc[c] = __builtin_amdgcn_mfma_f32_16x16x1f32(wu, f[c], acc[c], 0, 0, 0);
                 }
             };
             // The scheduling fences keep each group of loads ahead of the arithmetic of the
             // half-batches before it; left alone, the compiler sinks the loads to just before
             // their first use and every half-batch waits out the full memory latency.
-            f32x4 wr[D];
+            f32x4 wr[D][(HE + 3) / 4];
             u32x4 xr[D][H];
             issue(0, wr[0], xr[0], false);                        // the first gathers leave before the weights are in
             __builtin_amdgcn_sched_barrier(0);
@@ -365,15 +402,16 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
             // one wavefront writes and reads this part of LDS, and LDS operations of a wavefront
             // complete in order: no barrier between the workgroup's wavefronts is needed
             __builtin_amdgcn_wave_barrier();
-            wr[0] = sw[lane & 15];
 #pragma unroll
-            for (int k = 1; k < D - 1; ++k) issue(k * H, wr[k], xr[k], true);
-            for (int j = 0; j < mc; j += D * H) {
+            for (int t = 0; t < (HE + 3) / 4; ++t) wr[0][t] = sw[t * G + (lane & 15)];
+#pragma unroll
+            for (int k = 1; k < D - 1; ++k) issue(k * HE, wr[k], xr[k], true);
+            for (int j = 0; j < mc; j += D * HE) {
 #pragma unroll
                 for (int k = 0; k < D; ++k) {
-                    issue(j + (D - 1 + k) * H, wr[(D - 1 + k) % D], xr[(D - 1 + k) % D], true);
+                    issue(j + (D - 1 + k) * HE, wr[(D - 1 + k) % D], xr[(D - 1 + k) % D], true);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (k == 0 || j + k * H < mc) add_rows(wr[k], xr[k]);
+                    if (k == 0 || j + k * HE < mc) add_rows(wr[k], xr[k]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -383,13 +421,17 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
         const i32x4 my_rows = *reinterpret_cast<GlobalInt4Ptr>(reinterpret_cast<uintptr_t>(b.rows + cell * G + 4 * (lane >> 4)));
         const int row_of[4] = {my_rows.x, my_rows.y, my_rows.z, my_rows.w};
 #pragma unroll
-        for (int g = 0; g < 16; ++g) {
+        for (int g = 0; g < 4 * NB; ++g) {                        // g / 4: feature block, g % 4: row
             const int row = row_of[g & 3];
             if (row < 0) continue;
             float* dst = C + (size_t)row * ldc + VEC * (16 * (g >> 2) + (lane & 15));
 #pragma unroll
             for (int i = 0; i < VEC; i += 4) {
                 f32x4 o = {acc[i][g], acc[i + 1][g], acc[i + 2][g], acc[i + 3][g]};
+#pragma unroll
+                for (int e = 1; e < E; ++e)
+                    o += f32x4{acc[i][g + 4 * NB * e], acc[i + 1][g + 4 * NB * e], acc[i + 2][g + 4 * NB * e],
+                               acc[i + 3][g + 4 * NB * e]};
                 if (accumulate) o += *reinterpret_cast<const f32x4*>(dst + i);
                 __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(dst + i));
             }
@@ -577,8 +619,11 @@ int cells_build(const lf_bucket_desc& b, const int32_t* d_meta, int64_t num_rows
 int cells_launch(const LfCellBucket* d_buckets, int n_buckets, int grid, int b_dtype, const void* B, float* C,
                  int feat, int ldb, int ldc, int accumulate, hipStream_t s) {
     if (n_buckets <= 0 || grid <= 0) return LF_OK;
-    LF_REQUIRE(b_dtype == LF_DTYPE_F32, LF_ERR_UNSUPPORTED, "cells are built for fp32 operands only");
-    spmm_cell_kernel<float><<<grid, 64 * kCellTileCells, 0, s>>>(d_buckets, n_buckets, B, C, feat, ldb, ldc, accumulate);
+    LF_REQUIRE(b_dtype == LF_DTYPE_F32 && (feat == 256 || feat == 128), LF_ERR_UNSUPPORTED,
+               "cells are built for 128 or 256 fp32 features per pass");
+    const dim3 wg(64 * kCellTileCells);
+    if (feat == 256) spmm_cell_kernel<float, 64><<<grid, wg, 0, s>>>(d_buckets, n_buckets, B, C, feat, ldb, ldc, accumulate);
+    else spmm_cell_kernel<float, 32><<<grid, wg, 0, s>>>(d_buckets, n_buckets, B, C, feat, ldb, ldc, accumulate);
     LF_HIP(hipGetLastError());
     return LF_OK;
 }

@@ -1413,12 +1413,13 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             std::vector<int> chosen;
             for (size_t i = 0; i < cand.size(); ++i)
                 if (h_rg[3 * i + 1] > 0 && h_rg[3 * i] * 100 <= h_rg[3 * i + 1] * kRowGroupMaxPercent) chosen.push_back(cand[i]);
-            // One 16-byte load per lane covers a row of B (256 fp32 or 512 bf16 features): the
-            // chosen buckets are rewritten as cells of rows that are neighbours in up to three
-            // directions where that structure is found, else four consecutive rows at a time.
-            // (fp32 B only: with bf16 the 8 accumulator tiles of a 512-feature row leave room for
-            // one wavefront per SIMD, and the cells measured slower than the row groups)
-            if (!chosen.empty() && lpr == 64 && ch == 1 && b_dtype == LF_DTYPE_F32 && !(env && env[0] == '4')) {
+            // fp32 B, one 16-byte load per lane and 32 or 64 lanes per row of B (128 or 256
+            // features per pass): the chosen buckets are rewritten as cells of rows that are
+            // neighbours in up to three directions where that structure is found, else four
+            // consecutive rows at a time (as are all other operand shapes: the cells measured
+            // slower there).
+            const bool cells_fit = ch == 1 && (lpr == 64 || lpr == 32) && b_dtype == LF_DTYPE_F32;
+            if (!chosen.empty() && cells_fit && !(env && env[0] == '4')) {
                 std::vector<int> rest;
                 for (int k : chosen) {
                     LfCellBucket cb{};

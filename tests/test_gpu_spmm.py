@@ -339,30 +339,32 @@ def grid_stencil(rng, dims, reach=1):
     return MTX.from_coo(rows, cols, (n, n), data=rng.uniform(-1, 1, size=len(rows)).astype(np.float32))
 
 
-@pytest.mark.parametrize("feat,windows", [(256, 1), (512, 2)])
-def test_grid_stencils_are_served_as_cells(fa, torch, feat, windows, monkeypatch):
-    """fp32 B, 256 features per pass: buckets of a stencil become 16-row cells (neighbours in
-    every direction of the grid, found from the column differences) on the matrix cores; the
-    product is the plain path's to rounding and within the bound of the float64 oracle."""
+@pytest.mark.parametrize("feat,windows,b_dtype", [(256, 1, "f32"), (512, 2, "f32"), (128, 1, "f32"), (256, 2, "f32"),
+                                                  (512, 4, "f32")])
+def test_grid_stencils_are_served_as_cells(fa, torch, feat, windows, b_dtype, monkeypatch):
+    """fp32 B, 128 or 256 features per pass: buckets of a stencil become 16-row cells
+    (neighbours in every direction of the grid, found from the column differences) on the
+    matrix cores; the product is the plain path's to rounding and within the bound of the
+    float64 oracle."""
     rng = np.random.default_rng(77 + feat)
     for g, widths in ((grid_stencil(rng, (37, 29, 23)), [[8, 16, 32]]),        # 27 points, ragged cell edges
                       (grid_stencil(rng, (150, 131)), [[4, 8, 16]]),           # 9 points, two strides
                       (grid_stencil(rng, (64, 40, 16)), [[32]]),               # one bucket for faces and interior
                       (banded_matrix(rng, 9001, 10), [[8, 16, 32]])):          # one stride
-        C1, info = check(fa, torch, g, widths, feat, "f32", seed=feat, windows=windows)
+        C1, info = check(fa, torch, g, widths, feat, b_dtype, seed=feat, windows=windows)
         assert info["cell_buckets"] >= 1, (widths, info)
         monkeypatch.setenv("LF_ROW_GROUPS", "4")
-        C4, info4 = check(fa, torch, g, widths, feat, "f32", seed=feat, windows=windows)
+        C4, info4 = check(fa, torch, g, widths, feat, b_dtype, seed=feat, windows=windows)
         monkeypatch.setenv("LF_ROW_GROUPS", "0")
-        C0, info0 = check(fa, torch, g, widths, feat, "f32", seed=feat, windows=windows)
+        C0, info0 = check(fa, torch, g, widths, feat, b_dtype, seed=feat, windows=windows)
         monkeypatch.delenv("LF_ROW_GROUPS")
         assert info4["cell_buckets"] == 0 and info4["row_group_buckets"] >= 1
         assert info0["row_group_buckets"] == 0
-        # same terms per row in ascending column order on all three paths: they differ only in
-        # the rounding of fused multiply-adds (|a|, |b| < 1, at most 27 terms)
+        # same terms per row on all three paths (the cells add them as one or two interleaved
+        # partial sums): they differ only in rounding (|a|, |b| < 1, at most 27 terms)
         assert np.abs(C1 - C0).max() <= 2e-5 and np.abs(C4 - C0).max() <= 2e-5
     g = skewed_matrix(rng, 20000, 30000, mean_deg=20, heavy_rows=0)
-    _, info = check(fa, torch, g, [[8, 16, 32, 64]], feat, "f32", seed=feat, windows=windows)
+    _, info = check(fa, torch, g, [[8, 16, 32, 64]], feat, b_dtype, seed=feat, windows=windows)
     assert info["cell_buckets"] == 0
 
 
