@@ -494,8 +494,8 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
                 for (int e = 1; e < E; ++e)
                     o += f32x4{acc[i][g + 4 * NB * e], acc[i + 1][g + 4 * NB * e], acc[i + 2][g + 4 * NB * e],
                                acc[i + 3][g + 4 * NB * e]};
-                if (accumulate) o += *reinterpret_cast<const f32x4*>(dst + i);
-                __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(dst + i));
+                if (accumulate & kAccumulateC) o += *reinterpret_cast<const f32x4*>(dst + i);
+                store_f32x4(dst + i, o, accumulate & kStreamC);
             }
         }
         }

@@ -381,7 +381,7 @@ __device__ __forceinline__ void run_zero_tile(const Group& g, long long tile, co
     const int n = (int)min((long long)g.rows_per_tile, g.n_items - e0);
     Acc<CH, VEC> zero;
     zero.clear();
-    for (int r = sw; r < n; r += SW) store_row<LPR, CH, VEC>(a.C, g.rows[e0 + r], ln, zero, 0);
+    for (int r = sw; r < n; r += SW) store_row<LPR, CH, VEC>(a.C, g.rows[e0 + r], ln, zero, a.accumulate & kStreamC);
 }
 
 // One chunk of a heavy source row: the workgroup's sub-waves take consecutive slices of
@@ -764,7 +764,7 @@ csr_spmm_kernel(const int32_t* __restrict__ indptr, const int32_t* __restrict__ 
         Acc<CH, VEC> acc;
         acc.clear();
         stream_slots<LPR, CH, BT>(indices, values, lo, hi - lo, a.B, ln, acc);
-        store_row<LPR, CH, VEC>(a.C, (int)r, ln, acc, 0);
+        store_row<LPR, CH, VEC>(a.C, (int)r, ln, acc, kStreamC);
     }
 }
 
@@ -1056,6 +1056,7 @@ struct lf_spmm_plan {
         int cell_begin = 0, n_cell_buckets = 0, cell_grid = 0; // buckets rewritten as cells
         long long tiles = 0;
         int heavy_begin = 0, n_heavy = 0;
+        bool stream_c = false;       // store C past the caches (when this is the run's last partition)
     };
     std::vector<Launch> launches;
     MergedBucket* d_merged = nullptr;   // row-group buckets, grouped by partition
@@ -1492,6 +1493,15 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         std::vector<int> mine;
         for (int k = 0; k < num_buckets; ++k)
             if (h_buckets[k].part == p && h_buckets[k].num_ell_rows > 0) mine.push_back(k);
+        // Streaming stores leave the caches to B, but a launch whose rows are mostly short is
+        // made of stores as much as of gathers and loses by them: 2.45M-row graph (33 entries per
+        // row) 6.23 -> 6.13 ms, 500k x 2M matrix (most rows 2-4 entries) 1.46 -> 1.53 ms.
+        long long rows_wide = 0, rows_all = 0;
+        for (int k : mine) {
+            rows_all += h_buckets[k].num_ell_rows;
+            if (h_buckets[k].width >= kStreamMinWidth) rows_wide += h_buckets[k].num_ell_rows;
+        }
+        L.stream_c = rows_wide * 2 >= rows_all;
         L.heavy_begin = mine.empty() ? 0 : heavy_base[mine.front()];
         L.n_heavy = mine.empty() ? 0 : heavy_base[mine.back() + 1] - L.heavy_begin;
         for (int k : mine) {
@@ -1669,7 +1679,7 @@ int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t str
             LaunchArgs a{};
             a.groups = plan->d_groups + L.group_begin;
             a.n_groups = L.n_groups;
-            a.accumulate = p > 0 ? 1 : 0;
+            a.accumulate = (p > 0 ? kAccumulateC : 0) | (p + 1 == plan->num_parts && L.stream_c ? kStreamC : 0);
             a.feat = plan->feat;
             a.ldb = a.ldc = ld;
             a.B = (const char*)d_B + (size_t)w * plan->feat * b_elem;

@@ -78,7 +78,8 @@ struct Group {
 struct LaunchArgs {
     const Group* groups;
     int n_groups;
-    int accumulate;               // 0: C = result, 1: C += result
+    int accumulate;               // bit 0: C += result instead of C = result; bit 1 (kStreamC): no later
+                                  // launch of the run reads these rows of C again
     int feat;                     // N: features computed by the launch
     int ldb, ldc;                 // row strides of B and C in elements (N, or more for a feature window)
     int pad_;
@@ -160,21 +161,36 @@ __device__ __forceinline__ void gather_fma(const void* B, const Lane<LPR, CH, De
             for (int i = 0; i < VEC; ++i) acc.v[c][i] = fmaf(val[u], x[u][c][i], acc.v[c][i]);
 }
 
+// flags: LaunchArgs::accumulate.  Rows that nothing reads again in this run are stored
+// non-temporally where the launch's rows are mostly wide, which leaves the caches to B (2.45M-row
+// graph, N = 128: 6.23 -> 6.13 ms); rows that a later column partition adds to stay cached
+// (170k-row graph, two partitions: streaming them costs 7 %).
+constexpr int kAccumulateC = 1, kStreamC = 2;
+constexpr int kStreamMinWidth = 16;      // a launch streams C when at least half of its ELL rows are this wide
+typedef float lf_f32x4 __attribute__((ext_vector_type(4)));
+
+// 16 bytes to global memory, streamed or not by a run-time flag.  The streaming store goes
+// through a global-memory pointer made from the address as an integer: with the same pointer in
+// both branches the compiler folds the two stores into one ordinary store.
+__device__ __forceinline__ void store_f32x4(float* dst, lf_f32x4 o, bool stream) {
+    if (stream)
+        __builtin_nontemporal_store(o, reinterpret_cast<lf_f32x4 __attribute__((address_space(1)))*>(reinterpret_cast<uintptr_t>(dst)));
+    else
+        *reinterpret_cast<lf_f32x4*>(dst) = o;
+}
+
 template <int LPR, int CH, int VEC>
 __device__ __forceinline__ void store_row(float* C, int row, const Lane<LPR, CH, VEC>& ln,
-                                          const Acc<CH, VEC>& acc, int accumulate) {
+                                          const Acc<CH, VEC>& acc, int flags) {
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         if (!ln.on[c]) continue;
         float* dst = C + (size_t)row * ln.ldc + ln.f[c];
 #pragma unroll
         for (int i = 0; i < VEC; i += 4) {
-            float4 o = make_float4(acc.v[c][i], acc.v[c][i + 1], acc.v[c][i + 2], acc.v[c][i + 3]);
-            if (accumulate) {
-                const float4 old = *reinterpret_cast<const float4*>(dst + i);
-                o.x += old.x; o.y += old.y; o.z += old.z; o.w += old.w;
-            }
-            *reinterpret_cast<float4*>(dst + i) = o;
+            lf_f32x4 o = {acc.v[c][i], acc.v[c][i + 1], acc.v[c][i + 2], acc.v[c][i + 3]};
+            if (flags & kAccumulateC) o += *reinterpret_cast<const lf_f32x4*>(dst + i);
+            store_f32x4(dst + i, o, flags & kStreamC);
         }
     }
 }
