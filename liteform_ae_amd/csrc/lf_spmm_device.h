@@ -79,7 +79,8 @@ struct LaunchArgs {
     const Group* groups;
     int n_groups;
     int accumulate;               // bit 0: C += result instead of C = result; bit 1 (kStreamC): no later
-                                  // launch of the run reads these rows of C again
+                                  // launch of the run reads these rows of C again; bit 2 (kStreamSlabs):
+                                  // the slabs are too large to be worth caching
     int feat;                     // N: features computed by the launch
     int ldb, ldc;                 // row strides of B and C in elements (N, or more for a feature window)
     int pad_;
@@ -165,7 +166,7 @@ __device__ __forceinline__ void gather_fma(const void* B, const Lane<LPR, CH, De
 // non-temporally where the launch's rows are mostly wide, which leaves the caches to B (2.45M-row
 // graph, N = 128: 6.23 -> 6.13 ms); rows that a later column partition adds to stay cached
 // (170k-row graph, two partitions: streaming them costs 7 %).
-constexpr int kAccumulateC = 1, kStreamC = 2;
+constexpr int kAccumulateC = 1, kStreamC = 2, kStreamSlabs = 4;
 constexpr int kStreamMinWidth = 16;      // a launch streams C when at least half of its ELL rows are this wide
 typedef float lf_f32x4 __attribute__((ext_vector_type(4)));
 
@@ -177,6 +178,15 @@ __device__ __forceinline__ void store_f32x4(float* dst, lf_f32x4 o, bool stream)
         __builtin_nontemporal_store(o, reinterpret_cast<lf_f32x4 __attribute__((address_space(1)))*>(reinterpret_cast<uintptr_t>(dst)));
     else
         *reinterpret_cast<lf_f32x4*>(dst) = o;
+}
+
+// 16 bytes of a slab, streamed or not (same construction as store_f32x4)
+typedef int lf_i32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ lf_i32x4 load_i32x4(const void* src, bool stream) {
+    if (stream)
+        return __builtin_nontemporal_load(
+            reinterpret_cast<const lf_i32x4 __attribute__((address_space(1)))*>(reinterpret_cast<uintptr_t>(src)));
+    return *reinterpret_cast<const lf_i32x4*>(src);
 }
 
 template <int LPR, int CH, int VEC>
