@@ -49,11 +49,17 @@ __device__ __forceinline__ void stream_slots(const int32_t* __restrict__ cols, c
     constexpr int U = kUnroll < LPR ? kUnroll : LPR;
     if (total <= 0) return;
     const int c_first = cols[base];
+    // the next batch of slots is requested before the current one is walked: a slab is read
+    // once, so each of these loads waits out the full memory latency
+    int next_c = ln.sl < total ? cols[base + ln.sl] : c_first;
+    float next_v = ln.sl < total ? (vals ? vals[base + ln.sl] : 1.f) : 0.f;
     for (int off = 0; off < total; off += LPR) {
-        const int idx = off + ln.sl;
+        const int my_c = next_c;
+        const float my_v = next_v;
+        const int idx = off + LPR + ln.sl;
         const bool have = idx < total;
-        const int my_c = have ? cols[base + idx] : c_first;
-        const float my_v = have ? (vals ? vals[base + idx] : 1.f) : 0.f;
+        next_c = have ? cols[base + idx] : c_first;
+        next_v = have ? (vals ? vals[base + idx] : 1.f) : 0.f;
         const int cnt = min(LPR, total - off);
         for (int j = 0; j < cnt; j += U) {
             int c[U];
