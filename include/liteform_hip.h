@@ -221,7 +221,7 @@ int lf_hyb_build(const int32_t* d_indptr, const int32_t* d_indices, const float*
  * At creation, buckets of 8..64-slot rows whose neighbouring rows hold mostly the same columns
  * (stencils, banded and block-structured matrices) are rewritten inside the plan so that one
  * read of a B row serves several output rows: as groups of four consecutive rows with merged
- * column lists (about 21 bytes per merged entry), or - float32 B, 256 features per pass - as
+ * column lists (about 21 bytes per merged entry), or - float32 B, 128 or 256 features per pass - as
  * cells of 16 rows that are neighbours in up to three directions of the underlying grid (the
  * directions are read off the column differences of sampled rows; 68 bytes per merged entry),
  * accumulated with the fp32 outer-product matrix instruction.  This costs plan time and memory
