@@ -480,7 +480,8 @@ spmm_partition_kernel(LaunchArgs a) {
     }
 }
 
-// Adds the partial rows of every heavy source row in chunk order and writes the row.
+// Adds the partial rows of every heavy source row in chunk order and writes the row (rows with
+// more than kWideFinalPartials partial rows are left to spmm_finalize_wide_kernel).
 template <int LPR, int CH, typename BT>
 __global__ void __launch_bounds__(kWG)
 spmm_finalize_kernel(const HeavyRow* __restrict__ heavy, int n_heavy, LaunchArgs a) {
@@ -490,6 +491,7 @@ spmm_finalize_kernel(const HeavyRow* __restrict__ heavy, int n_heavy, LaunchArgs
     const Lane<LPR, CH, VEC> ln(sl, a.feat, a.ldb, a.ldc);
     for (int h = blockIdx.x * SW + sw; h < n_heavy; h += gridDim.x * SW) {
         const HeavyRow hr = heavy[h];
+        if (hr.n_partials > kWideFinalPartials) continue;
         Acc<CH, VEC> acc;
         acc.clear();
         for (int k = 0; k < hr.n_partials; ++k) {
@@ -502,6 +504,65 @@ spmm_finalize_kernel(const HeavyRow* __restrict__ heavy, int n_heavy, LaunchArgs
             }
         }
         store_row<LPR, CH, VEC>(a.C, hr.row, ln, acc, a.accumulate);
+    }
+}
+
+// The same for rows with many partial rows (dense rows cut into short chunks): one workgroup per
+// row, sub-wave s adds partial rows s, s + SW, s + 2 SW, ... four at a time, and the sub-waves'
+// sums are added in sub-wave order - a fixed order, so the result does not depend on scheduling.
+template <int LPR, int CH, typename BT>
+__global__ void __launch_bounds__(kWG)
+spmm_finalize_wide_kernel(const HeavyRow* __restrict__ heavy, int n_heavy, LaunchArgs a) {
+    constexpr int VEC = Dense<BT>::kVec;
+    constexpr int SW = kWG / LPR;
+    constexpr int U = 4;
+    __shared__ float s_red[kWG * CH * VEC];
+    const int sw = threadIdx.x / LPR, sl = threadIdx.x % LPR;
+    const Lane<LPR, CH, VEC> ln(sl, a.feat, a.ldb, a.ldc);
+    const int h = blockIdx.x;
+    if (h >= n_heavy) return;
+    const HeavyRow hr = heavy[h];
+    if (hr.n_partials <= kWideFinalPartials) return;
+    Acc<CH, VEC> acc;
+    acc.clear();
+    for (int k0 = sw; k0 < hr.n_partials; k0 += SW * U) {
+        float x[U][CH][VEC];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = min(k0 + u * SW, hr.n_partials - 1);      // (clamped loads, masked below)
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const float* src = a.partials + (size_t)(hr.partial_begin + k) * a.feat + (ln.on[c] ? ln.f[c] : 0);
+#pragma unroll
+                for (int i = 0; i < VEC; i += 4) {
+                    const float4 v = *reinterpret_cast<const float4*>(src + i);
+                    x[u][c][i] = v.x; x[u][c][i + 1] = v.y; x[u][c][i + 2] = v.z; x[u][c][i + 3] = v.w;
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (k0 + u * SW >= hr.n_partials) break;
+#pragma unroll
+            for (int c = 0; c < CH; ++c)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc.v[c][i] += x[u][c][i];
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) s_red[((sw * CH + c) * LPR + sl) * VEC + i] = acc.v[c][i];
+    __syncthreads();
+    if (sw == 0) {
+        Acc<CH, VEC> sum;
+        sum.clear();
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+            for (int s2 = 0; s2 < SW; ++s2)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) sum.v[c][i] += s_red[((s2 * CH + c) * LPR + sl) * VEC + i];
+        store_row<LPR, CH, VEC>(a.C, hr.row, ln, sum, a.accumulate);
     }
 }
 
@@ -936,14 +997,14 @@ validate_bucket_kernel(const int32_t* __restrict__ rows, const int32_t* __restri
 // partials are private and are summed in chunk order.
 __global__ void __launch_bounds__(256)
 plan_chunks_kernel(const int32_t* __restrict__ rows, const int32_t* __restrict__ meta,
-                   long long n_rows, int log_w, int* __restrict__ counters,
+                   const int32_t* __restrict__ cols, long long n_rows, int log_w, int* __restrict__ counters,
                    Chunk* __restrict__ chunks, HeavyRow* __restrict__ heavy,
-                   int partial_base, int heavy_base, int chunk_slots) {
+                   int partial_base, int heavy_base, int chunk_slots, long long dense_min_slots) {
     const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     const int lane = threadIdx.x & 63;
-    int seg = 0, n_chunks = 0;
-    bool split = false;
-    const int rows_per_chunk = max(1, chunk_slots >> log_w);
+    int seg = 0, n_chunks = 0, cs = chunk_slots;
+    long long total = 0;
+    bool split = false, dense = false;
     if (e < n_rows) {
         const int m = meta[e];
         if (m < 0) {
@@ -951,10 +1012,17 @@ plan_chunks_kernel(const int32_t* __restrict__ rows, const int32_t* __restrict__
         } else {
             seg = (int)((uint32_t)m >> kMetaLenBits);
             split = seg > 1;
-            if (((long long)seg << log_w) > kCoopSlots) n_chunks = (seg + rows_per_chunk - 1) / rows_per_chunk;
+            if (((long long)seg << log_w) > kCoopSlots) {
+                total = ((long long)(seg - 1) << log_w) + (meta[e + seg - 1] & kMetaLenMask);
+                dense = total >= dense_min_slots;
+                if (dense) cs = kDenseChunkSlots;
+                n_chunks = (int)((total + cs - 1) / cs);
+            }
         }
     }
-    if (__ballot(split) != 0 && lane == 0) counters[3] = 1;
+    if (__ballot(dense) != 0 && lane == 0) atomicOr(&counters[3], 2);
+    if (__ballot(n_chunks > kWideFinalPartials) != 0 && lane == 0) atomicOr(&counters[3], 4);
+    if (__ballot(split) != 0 && lane == 0) atomicOr(&counters[3], 1);
     // ranges of the tables: one atomic per counter and wavefront (a matrix of long rows has
     // a cooperative row in every lane)
     const bool several = n_chunks > 1;
@@ -982,17 +1050,16 @@ plan_chunks_kernel(const int32_t* __restrict__ rows, const int32_t* __restrict__
     const int c0 = base_c + incl_c - n_chunks;
     const int h = base_h + __popcll(votes & ((1ull << lane) - 1ull));
     const int p0 = base_p + incl_p - part;
-    const long long total = ((long long)(seg - 1) << log_w) + (meta[e + seg - 1] & kMetaLenMask);
     const int row = rows[e];
     for (int i = 0; i < n_chunks; ++i) {
-        const long long lo = (long long)i * rows_per_chunk << log_w;
-        const long long hi = min(total, (long long)(i + 1) * rows_per_chunk << log_w);
+        const long long lo = (long long)i * cs;
+        const long long hi = min(total, lo + cs);
         Chunk ck;
         ck.slot_begin = (e << log_w) + lo;
-        ck.n_slots = (int)(hi - lo);
+        ck.n_slots = (int)(hi - lo) | (dense ? kChunkDenseBit : 0);
         ck.partial = several ? partial_base + p0 + i : -1;
         ck.row = row;
-        ck.pad_ = 0;
+        ck.first_col = cols[ck.slot_begin];
         chunks[c0 + i] = ck;
     }
     if (several) heavy[heavy_base + h] = HeavyRow{row, partial_base + p0, n_chunks, 0};
@@ -1063,6 +1130,7 @@ struct lf_spmm_plan {
         long long tiles = 0;
         int heavy_begin = 0, n_heavy = 0;
         bool stream_c = false;       // store C past the caches (when this is the run's last partition)
+        bool wide_rows = false;      // some rows have more than kWideFinalPartials partial rows
     };
     std::vector<Launch> launches;
     bool stream_slabs = false;          // read the slabs non-temporally
@@ -1105,6 +1173,7 @@ using RowGroupFn = void (*)(const MergedBucket*, int, LaunchArgs);
 struct KernelSet {
     KernelFn tiles = nullptr;
     FinalFn finalize = nullptr;
+    FinalFn finalize_wide = nullptr;
     CsrFn csr = nullptr;
     RowGroupFn rowgroup = nullptr;   // one 16-byte chunk per lane only
 };
@@ -1117,10 +1186,12 @@ template <int LPR, int CH> void pick_kernels(int dtype, KernelSet* k) {
     if (dtype == LF_DTYPE_BF16) {
         k->tiles = spmm_partition_kernel<LPR, CH, bf16_t>;
         k->finalize = spmm_finalize_kernel<LPR, CH, bf16_t>;
+        k->finalize_wide = spmm_finalize_wide_kernel<LPR, CH, bf16_t>;
         k->csr = csr_spmm_kernel<LPR, CH, bf16_t>;
     } else {
         k->tiles = spmm_partition_kernel<LPR, CH, float>;
         k->finalize = spmm_finalize_kernel<LPR, CH, float>;
+        k->finalize_wide = spmm_finalize_wide_kernel<LPR, CH, float>;
         k->csr = csr_spmm_kernel<LPR, CH, float>;
     }
 }
@@ -1241,7 +1312,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     int* d_zero_count = d_counters + 4 * num_buckets;
     int* d_flags = d_counters + 4 * (num_buckets + 1);   // validate_bucket_kernel, derive_meta_kernel
     std::vector<int> h_counters((size_t)n_counters, 0);
-    std::vector<int> is_multi((size_t)num_buckets, 0);
+    std::vector<int> is_multi((size_t)num_buckets, 0), has_dense((size_t)num_buckets, 0), has_wide((size_t)num_buckets, 0);
     struct ChunkCount { int chunks = 0, heavy = 0, partials = 0; };
     std::vector<ChunkCount> counts((size_t)num_buckets);
     auto clear_counters = [&]() {
@@ -1265,11 +1336,19 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
     // 500k x 2M matrix 1.457 -> 1.443); those of a small one are worth keeping between products
     // (170k-row graph, 6 MB of slabs: 0.073 ms cached, 0.076 ms streamed).
     plan->stream_slabs = total_slots >= kLargeMatrixSlots;
+    const char* env_dense = getenv("LF_DENSE_ROWS");       // "0": dense rows are chunked like the other long rows
+    // (where the memory-side cache holds the partition's part of B anyway there is nothing to order)
+    const long long cols_p = lf::ceil_div(num_cols, num_parts);
+    const bool b_is_cached = cols_p * feat_size * (b_dtype == LF_DTYPE_BF16 ? 2 : 4) <= kDenseMinBBytes;
+    const long long dense_min_slots = (env_dense && env_dense[0] == '0') || b_is_cached
+                                          ? (1ll << 62)
+                                          : std::max<long long>(kDenseRowMinSlots, cols_p / kDenseRowShare);
     auto launch_plan_chunks = [&](int k, Chunk* out, HeavyRow* hout, int partial_base, int heavy_base) {
         const lf_bucket_desc& b = h_buckets[k];
         const int grid = (int)((b.num_ell_rows + 255) / 256);
-        plan_chunks_kernel<<<grid, 256, 0, s>>>(b.d_rows, meta[k], b.num_ell_rows, lf::ilog2(b.width),
-                                                d_counters + 4 * k, out, hout, partial_base, heavy_base, chunk_slots);
+        plan_chunks_kernel<<<grid, 256, 0, s>>>(b.d_rows, meta[k], b.d_cols, b.num_ell_rows, lf::ilog2(b.width),
+                                                d_counters + 4 * k, out, hout, partial_base, heavy_base, chunk_slots,
+                                                dense_min_slots);
         return hipGetLastError();
     };
     LF_TRY_HIP(clear_counters());
@@ -1316,7 +1395,9 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         counts[k].chunks = h_counters[4 * k + 0];
         counts[k].heavy = h_counters[4 * k + 1];
         counts[k].partials = h_counters[4 * k + 2];
-        is_multi[k] = h_counters[4 * k + 3];
+        is_multi[k] = h_counters[4 * k + 3] & 1;
+        has_dense[k] = (h_counters[4 * k + 3] >> 1) & 1;
+        has_wide[k] = (h_counters[4 * k + 3] >> 2) & 1;
     }
 
     // ---- chunk tables, heavy-row table (grouped by bucket, hence by partition) and partial rows
@@ -1370,6 +1451,23 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
         if (h_counters[4 * k] != counts[k].chunks || h_counters[4 * k + 1] != counts[k].heavy ||
             h_counters[4 * k + 2] != counts[k].partials)
             return bail(lf::fail(LF_ERR_INVALID, "bucket %d changed while the plan was being built", k));
+        if (has_dense[k]) {
+            // The chunks of dense rows go behind the others, in column order (ties: by row, so
+            // the order is the same in every plan): some thousands of records, sorted on the host.
+            std::vector<Chunk> h_chunks((size_t)counts[k].chunks);
+            LF_TRY_HIP(hipMemcpyAsync(h_chunks.data(), d_chunks[k], h_chunks.size() * sizeof(Chunk), hipMemcpyDeviceToHost, s));
+            LF_TRY_HIP(hipStreamSynchronize(s));
+            const auto mid = std::stable_partition(h_chunks.begin(), h_chunks.end(),
+                                                   [](const Chunk& x) { return (x.n_slots & kChunkDenseBit) == 0; });
+            std::sort(mid, h_chunks.end(), [](const Chunk& x, const Chunk& y) {
+                if (x.first_col != y.first_col) return x.first_col < y.first_col;
+                if (x.row != y.row) return x.row < y.row;
+                return x.slot_begin < y.slot_begin;
+            });
+            for (auto it = mid; it != h_chunks.end(); ++it) it->n_slots &= ~kChunkDenseBit;
+            LF_TRY_HIP(hipMemcpyAsync(d_chunks[k], h_chunks.data(), h_chunks.size() * sizeof(Chunk), hipMemcpyHostToDevice, s));
+            LF_TRY_HIP(hipStreamSynchronize(s));
+        }
     }
     n_zero = h_counters[4 * num_buckets];
     if (n_zero > 0) {
@@ -1513,6 +1611,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             if (h_buckets[k].width >= kStreamMinWidth) rows_wide += h_buckets[k].num_ell_rows;
         }
         L.stream_c = rows_wide * 2 >= rows_all;
+        for (int k : mine) L.wide_rows = L.wide_rows || has_wide[k];
         L.heavy_begin = mine.empty() ? 0 : heavy_base[mine.front()];
         L.n_heavy = mine.empty() ? 0 : heavy_base[mine.back() + 1] - L.heavy_begin;
         for (int k : mine) {
@@ -1521,9 +1620,9 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             g.type = kChunk;
             g.log_w = lf::ilog2(h_buckets[k].width);
             g.rows_per_tile = 1;
-            g.n_items = g.n_tiles = counts[k].chunks;
             g.cols = h_buckets[k].d_cols;
             g.vals = h_buckets[k].d_vals;
+            g.n_items = g.n_tiles = counts[k].chunks;       // (those of dense rows last, in column order)
             g.chunks = d_chunks[k];
             groups.push_back(g);
         }
@@ -1715,6 +1814,10 @@ int lf_spmm_run(lf_spmm_plan* plan, const void* d_B, float* d_C, lf_stream_t str
                 const int fgrid = std::min((L.n_heavy + sw - 1) / sw, 1024);
                 ks.finalize<<<fgrid, kWG, 0, s>>>(plan->d_heavy + L.heavy_begin, L.n_heavy, a);
                 LF_HIP(hipGetLastError());
+                if (L.wide_rows) {
+                    ks.finalize_wide<<<L.n_heavy, kWG, 0, s>>>(plan->d_heavy + L.heavy_begin, L.n_heavy, a);
+                    LF_HIP(hipGetLastError());
+                }
             }
         }
     }

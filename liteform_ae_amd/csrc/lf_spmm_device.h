@@ -37,6 +37,19 @@ constexpr int kCoopSlots = LF_COOP_SLOTS;    // a source row with more slab slot
 constexpr int kChunkSlots = LF_CHUNK_SLOTS;  // ... in chunks of this many slots (a whole number of ELL rows)
 constexpr int kChunkSlotsLarge = 8192;       // ... or this many, in a matrix of at least kLargeMatrixSlots slots
 constexpr long long kLargeMatrixSlots = 4ll << 20;
+// Dense rows: a row holding at least 1/kDenseRowShare of its partition's columns.  Several of
+// them read much the same rows of B, so they are cut into shorter chunks that are walked in
+// column order: the chunks in flight then cover a window of B that the memory-side cache holds,
+// and a row of B is fetched from HBM once for all of them.  500k x 2M matrix with 50 rows of
+// 100,000 entries, bf16 N = 512, ms per product by chunk size (whole workgroup per chunk):
+// 8192 unordered 1.46; ordered 8192 1.53, 4096 1.43, 2048 1.39, 1024 1.295, 512 1.30, 256 1.40,
+// 128 1.70; a sub-wave per chunk: 512 1.40, 256 1.37, 128 1.34, 64 1.44.  (Short enough for
+// the window to fit an XCD's L2 they would need far fewer chunks in flight than fill the GPU.)
+constexpr int kDenseRowShare = 32;
+constexpr int kDenseRowMinSlots = 4096;
+constexpr long long kDenseMinBBytes = 128ll << 20;   // ... in a partition whose part of B is larger than this
+constexpr int kDenseChunkSlots = 1024;
+constexpr int kWideFinalPartials = 64;       // rows with more partial rows are added up by a whole workgroup
 constexpr int kXcds = 8;
 constexpr int kPartBytesMax = 16384;   // LDS for per-ELL-row sums of a balanced segment tile at most
 constexpr int kUnroll = LF_UNROLL;  // B-row gathers in flight per sub-wave
@@ -45,13 +58,15 @@ constexpr int kMetaLenBits = 11;
 
 enum GroupType : int { kEll = 0, kSeg = 1, kZero = 2, kChunk = 3, kEllSeg = 4 };
 
+constexpr int kChunkDenseBit = 1 << 30;       // in Chunk::n_slots while the plan is built: a piece of a dense row
+
 struct Chunk {
     long long slot_begin;   // first slot, relative to the bucket's slab
     int n_slots;
     int partial;            // index of the partial row this chunk produces; < 0: the chunk is the
                             // whole source row and goes straight to C
     int row;                // source row
-    int pad_;
+    int first_col;          // column of the chunk's first slot (chunks of dense rows are ordered by it)
 };
 
 struct HeavyRow {

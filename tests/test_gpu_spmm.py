@@ -322,6 +322,41 @@ def mixed_band_matrix(rng, n):
     return MTX.from_coo(rows, cols, (n, n), data=rng.uniform(-1, 1, size=len(rows)).astype(np.float32))
 
 
+@pytest.mark.parametrize("feat,b_dtype,parts,nc", [(64, "f32", 1, 640_000), (128, "bf16", 1, 640_000),
+                                                   (256, "f32", 2, 320_000), (512, "bf16", 1, 160_000)])
+def test_dense_rows_are_walked_in_column_order(fa, torch, feat, b_dtype, parts, nc, monkeypatch):
+    """Rows holding a large share of the columns are cut into short chunks that are walked in
+    column order and added up by a whole workgroup; the product is the same (to rounding) as
+    with the chunks of ordinary long rows, and bit-reproducible.  (Only where a partition's
+    part of B is larger than the memory-side cache: 160 MB here.)"""
+    rng = np.random.default_rng(500 + feat)
+    nr = 3000
+    g = skewed_matrix(rng, nr, nc, mean_deg=6, heavy_rows=3, heavy_len=90_000)      # 88 chunks of 1024 per dense row
+    widths = fa.search_bucket_config(g, parts, fa.CostModelSettings(feat, parts, cost_model="gfx950"))
+    C1, info = check(fa, torch, g, widths, feat, b_dtype, seed=feat)
+    assert info["partial_rows"] >= 3 * 64                            # more than 64 a row: added up by a whole workgroup (one partition)
+    monkeypatch.setenv("LF_DENSE_ROWS", "0")
+    C0, info0 = check(fa, torch, g, widths, feat, b_dtype, seed=feat)
+    monkeypatch.delenv("LF_DENSE_ROWS")
+    assert info0["partial_rows"] < info["partial_rows"]
+    indptr, _, data = g.adj_tensors("csr")
+    row_abs = np.add.reduceat(np.abs(np.asarray(data, dtype=np.float64)), np.minimum(indptr[:-1], len(data) - 1))
+    row_abs[np.diff(indptr) == 0] = 0
+    assert (np.abs(C1 - C0) <= 2e-5 * row_abs[:, None] + 1e-30).all()
+
+
+def test_very_long_row_is_added_up_by_a_workgroup(fa, torch):
+    """A row of ~170,000 entries in a small matrix (B fits the memory-side cache, so nothing is
+    reordered): over 80 chunks of 2048 slots, more partial rows than a sub-wave adds up alone."""
+    rng = np.random.default_rng(77)
+    g = skewed_matrix(rng, 500, 300_000, mean_deg=5, heavy_rows=1, heavy_len=260_000)
+    widths = fa.search_bucket_config(g, 1, fa.CostModelSettings(32, 1, cost_model="gfx950"))
+    _, info = check(fa, torch, g, widths, 32, "f32", seed=3)
+    assert info["partial_rows"] > 64
+    _, info = check(fa, torch, g, widths, 96, "f32", seed=4)          # three 16-byte chunks per lane, one unused
+    assert info["partial_rows"] > 64
+
+
 def grid_stencil(rng, dims, reach=1):
     """Every point of a grid (first dimension fastest) coupled to its neighbours within `reach`
     in every direction: 9 columns per interior row in two dimensions, 27 in three."""
