@@ -226,6 +226,10 @@ int lf_hyb_build(const int32_t* d_indptr, const int32_t* d_indices, const float*
  * directions are read off the column differences of sampled rows; 68 bytes per merged entry),
  * accumulated with the fp32 outer-product matrix instruction.  This costs plan time and memory
  * only where a sample of the bucket shows at least 30 % fewer reads.
+ * Rows that hold at least 1/32 of their partition's columns (and 4096 entries), in a partition
+ * whose part of B is larger than 128 MB, are reduced in chunks of 1024 slots that are walked in
+ * column order, so that such rows share what the memory-side cache holds of B (LF_DENSE_ROWS=0
+ * in the environment at plan creation: chunked like any other long row).
  * feat_size must be a multiple of 32 (float32 B) or 64 (bf16 B), at most 1024.
  * ------------------------------------------------------------------------------------ */
 typedef struct lf_bucket_desc {
