@@ -98,6 +98,25 @@ def test_model_prefers_windows_only_where_b_outgrows_the_memory_side_cache():
             assert abs(ms / got - 1) < (0.30 if got >= 0.5 else 0.50), (key, shape, ms, got)
 
 
+def test_fewest_launches_win_among_shapes_within_two_percent():
+    assert pick_launch_shape({(1, 1): 1.00, (1, 2): 0.99, (2, 1): 0.985}) == (1, 1)
+    assert pick_launch_shape({(1, 1): 1.00, (1, 2): 0.97, (2, 1): 0.969}) == (1, 2)      # same launches: fewer partitions
+    assert pick_launch_shape({(1, 1): 1.10, (2, 2): 1.00, (1, 4): 1.015}) == (1, 4)
+    assert pick_launch_shape({(1, 1): 1.10, (2, 2): 1.00, (1, 4): 1.03}) == (2, 2)
+    assert pick_launch_shape({(3, 1): 2.0}) == (3, 1)
+
+
+def test_structured_matrices_take_the_feature_count_their_kernels_want():
+    from liteform_ae_amd.format_algos import _structured_windows, _window_candidates
+    want = {(64, "f32"): 1, (128, "f32"): 1, (256, "f32"): 1, (512, "f32"): 2, (1024, "f32"): 4, (384, "f32"): 1,
+            (256, "bf16"): 1, (512, "bf16"): 1}
+    for (feat, dt), w in want.items():
+        assert _structured_windows(feat, dt, _window_candidates(feat, dt)) == w, (feat, dt)
+    assert _window_candidates(128, "f32") == [1, 2] and _window_candidates(64, "f32") == [1]
+    assert _window_candidates(512, "bf16") == [1, 2, 4, 8]
+    assert _structured_windows(512, "f32", [1]) == 1             # only what the caller allows
+
+
 def test_model_argument_errors():
     stats = uniform_stats(1000, 8)
     with pytest.raises(ValueError):
