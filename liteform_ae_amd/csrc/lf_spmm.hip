@@ -1528,7 +1528,7 @@ int lf_spmm_create(lf_spmm_plan** out_plan, const lf_bucket_desc* h_buckets, int
             // neighbours in up to three directions where that structure is found, else four
             // consecutive rows at a time (as are all other operand shapes: the cells measured
             // slower there).
-            const bool cells_fit = ch == 1 && (lpr == 64 || lpr == 32) && b_dtype == LF_DTYPE_F32;
+            const bool cells_fit = (feat_size == 256 || feat_size == 128) && b_dtype == LF_DTYPE_F32;
             if (!chosen.empty() && cells_fit && !(env && env[0] == '4')) {
                 std::vector<int> rest;
                 for (int k : chosen) {

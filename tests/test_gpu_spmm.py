@@ -403,6 +403,15 @@ def test_grid_stencils_are_served_as_cells(fa, torch, feat, windows, b_dtype, mo
     assert info["cell_buckets"] == 0
 
 
+@pytest.mark.parametrize("feat", [96, 160, 224])
+def test_feature_counts_that_leave_lanes_unused_stay_with_row_groups(fa, torch, feat):
+    """160 features take 40 of 64 lanes: the lane layout of the 256-feature kernels, but not the
+    cells' (they want every lane of the row to hold features)."""
+    rng = np.random.default_rng(feat)
+    _, info = check(fa, torch, grid_stencil(rng, (30, 22, 17)), [[8, 16, 32]], feat, "f32", seed=feat)
+    assert info["cell_buckets"] == 0 and info["row_group_buckets"] >= 1
+
+
 @pytest.mark.parametrize("feat,b_dtype", [(32, "f32"), (64, "f32"), (128, "f32"), (256, "f32"), (256, "bf16"),
                                           (512, "bf16")])
 def test_rows_sharing_columns_are_served_in_groups(fa, torch, feat, b_dtype, monkeypatch):
