@@ -646,6 +646,8 @@ def row_overlap_device(g, max_samples: int = 8192) -> float:
     torch = _torch()
     lib = _lib.load()
     dev = _device_csr(g)
+    if dev.nnz == 0 or dev.num_rows < 2:
+        return 0.0
     out = np.zeros(2, dtype=np.int64)
     scratch = torch.empty(2, dtype=torch.int64, device="cuda")
     stride = max(1, dev.num_rows // max_samples)

@@ -45,6 +45,9 @@ def test_row_overlap_matches_numpy(fa):
         _lib.check(lib.lf_row_overlap(dev.indptr.data_ptr(), dev.indices.data_ptr(), dev.num_rows, stride,
                                       scratch.data_ptr(), _lib.np_ptr(out, C.c_int64), None))
         assert tuple(out) == overlap_numpy(g, stride)
+    assert fa.row_overlap_device(MTX.from_coo(np.array([], dtype=np.int32), np.array([], dtype=np.int32), (10, 10))) == 0.0
+    assert fa.predict_launch_shape(MTX.from_coo(np.array([], dtype=np.int32), np.array([], dtype=np.int32), (10, 10)), 64) == (1, 1)
+    assert fa.predict_launch_shape(MTX.from_coo(np.array([0]), np.array([0]), (1, 5)), 128)[0] == 1
     assert fa.row_overlap_device(make_workload("cfg4", 0.05).matrix) > 0.6      # 18 of 27 columns, less at the faces
     assert fa.row_overlap_device(skewed_matrix(rng, 20000, 200000, mean_deg=10)) < 0.01
 
