@@ -21,6 +21,7 @@ import sys
 import time
 
 import numpy as np
+import scipy.sparse as sp
 
 from .format_matrix_market import MTX
 
@@ -103,7 +104,17 @@ def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="
             time_bucket = time.perf_counter() - t0
 
             x = torch.ones((g.num_dst_nodes(), feat))                  # proc05:162
-            y_ndarray = g.dot(x.numpy()) if check_correctness else None
+            y_ndarray = None
+            if check_correctness:
+                # the expected product has to use the values the format is composed with: the
+                # matrix's own, or ones (the reference's matrices hold nothing else,
+                # format_matrix_market.py:63-64)
+                if keep_values:
+                    y_ndarray = g.dot(x.numpy())
+                else:
+                    indptr, indices, _ = g.adj_tensors("csr")
+                    ones = sp.csr_matrix((np.ones(len(indices), dtype=np.float32), indices, indptr), shape=g.coo_mtx.shape)
+                    y_ndarray = ones.dot(x.numpy())
             compose_ms = float("nan")
             try:
                 if keep_values:

@@ -257,6 +257,13 @@ def test_partition_chooser_and_driver_table(fa, torch, monkeypatch):
     assert list(df.columns[:8]) == ["name", "format", "feat_size", "num_parts", "time_select(s)",
                                     "time_num_parts(s)", "time_bucket(s)", "time_exe_our(ms)"]
     assert len(df) == 2 and (df["format"] == "CELL").all() and np.isfinite(df["time_exe_our(ms)"]).all()
+    # a matrix with values: the check compares with the values the format is composed with
+    # (ones by default, like the reference's matrices; the matrix's own with keep_values)
+    gw = skewed_matrix(rng, 2000, 2500, mean_deg=6, heavy_rows=1)
+    gw.name = "weighted"
+    for keep in (False, True):
+        df = driver.run_end_to_end([gw], feat_sizes=(64,), cost_model="gfx950", check_correctness=True, keep_values=keep)
+        assert np.isfinite(df["time_exe_our(ms)"]).all(), keep
 
 
 @pytest.mark.parametrize("feat,b_dtype,windows", [(128, "f32", 2), (256, "f32", 4), (512, "f32", 2), (256, "bf16", 2),
