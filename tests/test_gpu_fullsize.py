@@ -176,3 +176,28 @@ def test_launch_shape_model_on_the_headline_graph(big):
     best, table = fa.predict_launch_shape(g, 128, return_predictions=True)
     assert best == (1, 2)
     assert 5.0 < table[best] < 8.0            # predicted milliseconds (measured: 6.2)
+
+
+@pytest.mark.parametrize("feat,shapes", [(128, [(1, 1), (1, 2), (2, 1), (2, 2)]),
+                                         (256, [(1, 2), (1, 4), (2, 2), (2, 4)])])
+def test_model_pick_is_close_to_the_fastest_measured_shape(big, feat, shapes):
+    """The launch shape the model picks for the 2.45M-row graph, timed against its nearest
+    competitors (the shapes that were within a few percent of the fastest in the sweep the
+    model was fitted to): within 3 % of the fastest of them."""
+    wl, fa, torch = big
+    g = wl.matrix
+    pick = fa.predict_launch_shape(g, feat)
+    assert pick in shapes, pick
+    B = torch.rand((g.num_dst_nodes(), feat), device="cuda") - 0.5
+    C = torch.empty((g.num_src_nodes(), feat), device="cuda")
+    ms = {}
+    for p in sorted({s[0] for s in shapes}):
+        cfg = fa.search_bucket_config(g, p, fa.CostModelSettings(feat, p, cost_model="gfx950"))
+        fmt = fa.build_hyb_format_device(g, cfg)
+        for w in sorted({s[1] for s in shapes if s[0] == p}):
+            plan = fa.HybSpMM(fmt, feat, windows=w)
+            ms[(p, w)] = float(np.median(plan.time_ms(B, C, warmup=2, repeat=5)))
+            plan.close()
+        del fmt
+    assert ms[pick] <= 1.03 * min(ms.values()), (pick, ms)
+
