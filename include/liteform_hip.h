@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define LF_VERSION 100 /* 0.1.0 */
+#define LF_VERSION 110 /* 0.1.1 */
 
 #define LF_OK 0
 #define LF_ERR_INVALID (-1)     /* bad argument (null pointer, size, non power-of-two width ...) */
@@ -280,11 +280,36 @@ int lf_spmm_time_ms(lf_spmm_plan* plan, const void* d_B, float* d_C, int32_t war
                     int32_t repeat, void* d_flush, size_t flush_bytes, float* h_ms,
                     lf_stream_t stream);
 
+/* Structural check of CSR arrays that come from outside the library, on the GPU, before
+ * anything gathers through them (the reference hands its arrays to the generated kernel
+ * unchecked, format_algos.py:1729-1749).  LF_ERR_INVALID when the row pointer does not start at
+ * 0, decreases anywhere or does not end at nnz, or when a column index lies outside
+ * [0, num_cols).  *h_flags (optional) receives LF_CSR_CANONICAL when in addition the columns of
+ * every row ascend strictly (sorted, no duplicates) - the form scipy's coo.tocsr() produces
+ * (format_matrix_market.py:74-76) and lf_bucket_stats / lf_hyb_build expect, so that such
+ * arrays can be used as they are instead of going through lf_coo_to_csr - and
+ * LF_CSR_UNIT_VALUES when d_values (optional) holds nothing but 1.0, like every matrix of the
+ * reference (format_matrix_market.py:54, 63-64).  The block structure of a BSR matrix is
+ * checked the same way (rows and columns counted in blocks).  d_scratch: 16 bytes of device
+ * memory.  Synchronises the stream. */
+#define LF_CSR_CANONICAL 1
+#define LF_CSR_UNIT_VALUES 2
+int lf_csr_check(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values,
+                 int64_t num_rows, int64_t num_cols, int64_t nnz, void* d_scratch, int32_t* h_flags,
+                 lf_stream_t stream);
+
 /* Row-parallel CSR SpMM, the counterpart of bench_naive's kernel
- * (format_algos.py:1689-1755): C = A_csr . B with float32 values (NULL = ones). */
+ * (format_algos.py:1689-1755): C = A_csr . B with float32 values (NULL = ones).
+ * lf_csr_spmm runs lf_csr_check on the arrays first (d_scratch: its 16 bytes; the stream is
+ * synchronised for the verdict) and returns LF_ERR_INVALID without launching the product when
+ * they fail.  lf_csr_spmm_trusted is the same product without the check, for arrays that
+ * lf_csr_check has accepted or that lf_coo_to_csr produced: it only enqueues the kernel. */
 int lf_csr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values,
-                int64_t num_rows, int64_t num_cols, int32_t feat_size, int32_t b_dtype,
-                const void* d_B, float* d_C, lf_stream_t stream);
+                int64_t num_rows, int64_t num_cols, int64_t nnz, int32_t feat_size, int32_t b_dtype,
+                const void* d_B, float* d_C, void* d_scratch, lf_stream_t stream);
+int lf_csr_spmm_trusted(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values,
+                        int64_t num_rows, int64_t num_cols, int32_t feat_size, int32_t b_dtype,
+                        const void* d_B, float* d_C, lf_stream_t stream);
 
 /* COO -> canonical CSR on the GPU: entries sorted by (row, column), duplicates added up,
  * row pointer built - what the reference's container does with scipy's coo.tocsr() on every
@@ -302,10 +327,17 @@ int lf_coo_to_csr(const int32_t* d_coo_row, const int32_t* d_coo_col, const floa
  * (format_algos.py:1182-1643): Y = A_bsr . X with 32 x 32 fp16 blocks (scipy BSR layout:
  * indptr [num_block_rows + 1], indices [nnz blocks], data [nnz blocks][32][32] row-major),
  * X [num_block_cols * 32][feat] fp16, Y [num_block_rows * 32][feat] fp16, fp32 accumulation
- * (the reference accumulates in fp16).  feat_size must be a multiple of 8. */
+ * (the reference accumulates in fp16).  feat_size must be a multiple of 8.
+ * lf_bsr_spmm checks the block index arrays like lf_csr_check (d_scratch: 16 bytes of device
+ * memory; synchronises for the verdict) and returns LF_ERR_INVALID without launching the
+ * product when they fail; lf_bsr_spmm_trusted only enqueues the kernel, for arrays that have
+ * passed the check before. */
 int lf_bsr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const void* d_data,
-                int64_t num_block_rows, int64_t num_block_cols, int32_t block_size,
-                int32_t feat_size, const void* d_X, void* d_Y, lf_stream_t stream);
+                int64_t num_block_rows, int64_t num_block_cols, int64_t nnz_blocks, int32_t block_size,
+                int32_t feat_size, const void* d_X, void* d_Y, void* d_scratch, lf_stream_t stream);
+int lf_bsr_spmm_trusted(const int32_t* d_indptr, const int32_t* d_indices, const void* d_data,
+                        int64_t num_block_rows, int64_t num_block_cols, int32_t block_size,
+                        int32_t feat_size, const void* d_X, void* d_Y, lf_stream_t stream);
 
 #ifdef __cplusplus
 }

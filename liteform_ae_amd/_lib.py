@@ -26,6 +26,8 @@ LF_DTYPE_F32 = 0
 LF_DTYPE_BF16 = 1
 LF_COST_REFERENCE = 0
 LF_COST_GFX950 = 1
+LF_CSR_CANONICAL = 1
+LF_CSR_UNIT_VALUES = 2
 
 # LITEFORM_HIP_LIB points at another build of the same library (kernel tuning experiments)
 LIB_PATH = os.environ.get("LITEFORM_HIP_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)),
@@ -73,10 +75,13 @@ SIGNATURES = {
     "lf_spmm_set_windows": (C.c_int, [vp, C.c_int32]),
     "lf_spmm_info": (C.c_int, [vp, i64p]),
     "lf_spmm_time_ms": (C.c_int, [vp, vp, vp, C.c_int32, C.c_int32, vp, C.c_size_t, f32p, vp]),
-    "lf_csr_spmm": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int32, C.c_int32, vp, vp, vp]),
+    "lf_csr_check": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int64, vp, i32p, vp]),
+    "lf_csr_spmm": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_int32, vp, vp, vp, vp]),
+    "lf_csr_spmm_trusted": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int32, C.c_int32, vp, vp, vp]),
     "lf_coo_to_csr_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int64]),
     "lf_coo_to_csr": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int64, vp, C.c_size_t, vp, vp, vp, i64p, vp]),
-    "lf_bsr_spmm": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int32, C.c_int32, vp, vp, vp]),
+    "lf_bsr_spmm": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_int32, vp, vp, vp, vp]),
+    "lf_bsr_spmm_trusted": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, C.c_int32, C.c_int32, vp, vp, vp]),
 }
 
 _lock = threading.Lock()

@@ -103,9 +103,11 @@ bsr_spmm_kernel(const int32_t* __restrict__ indptr, const int32_t* __restrict__ 
 
 }  // namespace
 
-extern "C" int lf_bsr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const void* d_data,
-                           int64_t num_block_rows, int64_t num_block_cols, int32_t block_size,
-                           int32_t feat_size, const void* d_X, void* d_Y, lf_stream_t stream) {
+extern "C" {
+
+int lf_bsr_spmm_trusted(const int32_t* d_indptr, const int32_t* d_indices, const void* d_data,
+                        int64_t num_block_rows, int64_t num_block_cols, int32_t block_size,
+                        int32_t feat_size, const void* d_X, void* d_Y, lf_stream_t stream) {
     hipStream_t s = (hipStream_t)stream;
     LF_REQUIRE(block_size == kBs, LF_ERR_UNSUPPORTED, "only 32 x 32 blocks are supported (got %d)", block_size);
     LF_REQUIRE(num_block_rows >= 0 && num_block_rows < (1ll << 26) && num_block_cols >= 1 &&
@@ -122,3 +124,18 @@ extern "C" int lf_bsr_spmm(const int32_t* d_indptr, const int32_t* d_indices, co
     LF_HIP(hipGetLastError());
     return LF_OK;
 }
+
+int lf_bsr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const void* d_data,
+                int64_t num_block_rows, int64_t num_block_cols, int64_t nnz_blocks, int32_t block_size,
+                int32_t feat_size, const void* d_X, void* d_Y, void* d_scratch, lf_stream_t stream) {
+    LF_REQUIRE(num_block_rows >= 0 && num_block_rows < (1ll << 26) && num_block_cols >= 1 &&
+                   num_block_cols < (1ll << 26), LF_ERR_INVALID, "bad block shape");
+    // no gather before the block index arrays have passed
+    if (int rc = lf::csr_check(d_indptr, d_indices, nullptr, num_block_rows, num_block_cols, nnz_blocks, d_scratch, nullptr,
+                               "lf_bsr_spmm", (hipStream_t)stream))
+        return rc;
+    return lf_bsr_spmm_trusted(d_indptr, d_indices, d_data, num_block_rows, num_block_cols, block_size, feat_size,
+                               d_X, d_Y, stream);
+}
+
+}  // extern "C"

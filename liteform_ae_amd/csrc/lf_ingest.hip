@@ -5,6 +5,11 @@
 // lf_bucket_stats / lf_hyb_build.  Sorting and the segmented sum are plain library
 // primitives (rocPRIM radix sort and reduce-by-key on a 64-bit key row * cols + col); the
 // kernels written here only pack / unpack keys and locate the row boundaries.
+//
+// Also here: the structural check of CSR arrays that come from a caller (lf_csr_check), which
+// every entry point that gathers through caller-supplied CSR or BSR index arrays runs first,
+// and which tells an already canonical CSR (the fast path: no sort) from one that has to go
+// through the COO route.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -52,6 +57,48 @@ __global__ void row_pointer_kernel(const unsigned long long* __restrict__ keys, 
     indptr[r] = (int32_t)lo;
 }
 
+// One pass over the row pointer and one over the column indices.  out[0] is raised for
+// anything a gather must not meet: a row pointer that does not start at 0, decreases, or
+// does not end at nnz, or a column outside [0, num_cols).  out[1] counts the positions i > 0
+// with indices[i] <= indices[i - 1] ("descents"), out[2] the non-empty rows whose first
+// entry is such a position: the columns of every row ascend strictly (sorted, no
+// duplicates) exactly when the two counts are equal.  out[3] is raised when a value differs
+// from 1 (values == nullptr: not looked at).
+__global__ void __launch_bounds__(256)
+csr_check_kernel(const int32_t* __restrict__ indptr, const int32_t* __restrict__ indices,
+                 const float* __restrict__ values, long long rows, long long cols, long long nnz,
+                 unsigned int* __restrict__ out) {
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    const long long t0 = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    bool bad = false, not_one = false;
+    unsigned int descents = 0, boundary = 0;
+    for (long long r = t0; r < rows; r += stride) {
+        const long long lo = indptr[r], hi = indptr[r + 1];
+        bad |= lo < 0 || hi < lo || hi > nnz;
+        if (r == 0) bad |= lo != 0;
+        if (r == rows - 1) bad |= hi != nnz;
+        if (hi > lo && lo > 0 && lo < nnz && indices[lo] <= indices[lo - 1]) ++boundary;
+    }
+    for (long long i = t0; i < nnz; i += stride) {
+        const int c = indices[i];
+        bad |= (unsigned long long)(unsigned int)c >= (unsigned long long)cols;
+        if (i > 0 && c <= indices[i - 1]) ++descents;
+        if (values) not_one |= values[i] != 1.0f;
+    }
+    for (int d = 32; d > 0; d >>= 1) {
+        descents += __shfl_xor(descents, d);
+        boundary += __shfl_xor(boundary, d);
+    }
+    const bool any_bad = __ballot(bad) != 0;
+    const bool any_not_one = __ballot(not_one) != 0;
+    if ((threadIdx.x & 63) == 0) {
+        if (any_bad) out[0] = 1u;
+        if (any_not_one) out[3] = 1u;
+        if (descents) atomicAdd(&out[1], descents);
+        if (boundary) atomicAdd(&out[2], boundary);
+    }
+}
+
 struct IngestLayout {
     size_t keys_a, keys_b, vals_a, count, temp, temp_bytes, total;
 };
@@ -87,7 +134,45 @@ int key_bits_for(long long rows, long long cols) {
 
 }  // namespace
 
+namespace lf {
+
+int csr_check(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values, int64_t num_rows,
+              int64_t num_cols, int64_t nnz, void* d_scratch, int32_t* h_flags, const char* what, hipStream_t s) {
+    LF_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31) && num_cols >= 1 && num_cols < (1ll << 31), LF_ERR_INVALID,
+               "bad shape %lld x %lld", (long long)num_rows, (long long)num_cols);
+    LF_REQUIRE(nnz >= 0 && nnz < (1ll << 31), LF_ERR_UNSUPPORTED, "nnz must be below 2^31");
+    if (h_flags) *h_flags = LF_CSR_CANONICAL | (d_values ? LF_CSR_UNIT_VALUES : 0);
+    if (num_rows == 0) {
+        LF_REQUIRE(nnz == 0, LF_ERR_INVALID, "%s: a matrix without rows holds %lld entries", what, (long long)nnz);
+        return LF_OK;
+    }
+    LF_REQUIRE(d_indptr && (nnz == 0 || d_indices), LF_ERR_INVALID, "%s: null index array", what);
+    LF_REQUIRE(d_scratch && (uintptr_t)d_scratch % 4 == 0, LF_ERR_INVALID, "%s: the check needs 16 bytes of device scratch", what);
+    unsigned int* out = (unsigned int*)d_scratch;
+    LF_HIP(hipMemsetAsync(out, 0, 16, s));
+    const long long units = std::max<long long>(num_rows, nnz);
+    const int grid = (int)std::min<long long>((units + 255) / 256, 8192);
+    csr_check_kernel<<<grid, 256, 0, s>>>(d_indptr, d_indices, d_values, num_rows, num_cols, nnz, out);
+    LF_HIP(hipGetLastError());
+    unsigned int h[4] = {0, 0, 0, 0};
+    LF_HIP(hipMemcpyAsync(h, out, 16, hipMemcpyDeviceToHost, s));
+    LF_HIP(hipStreamSynchronize(s));
+    LF_REQUIRE(h[0] == 0, LF_ERR_INVALID,
+               "%s: the row pointer is not a non-decreasing sequence from 0 to nnz = %lld, or an index lies outside [0, %lld)",
+               what, (long long)nnz, (long long)num_cols);
+    if (h_flags) *h_flags = (h[1] == h[2] ? LF_CSR_CANONICAL : 0) | (d_values && h[3] == 0 ? LF_CSR_UNIT_VALUES : 0);
+    return LF_OK;
+}
+
+}  // namespace lf
+
 extern "C" {
+
+int lf_csr_check(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values, int64_t num_rows,
+                 int64_t num_cols, int64_t nnz, void* d_scratch, int32_t* h_flags, lf_stream_t stream) {
+    return lf::csr_check(d_indptr, d_indices, d_values, num_rows, num_cols, nnz, d_scratch, h_flags, "CSR arrays",
+                         (hipStream_t)stream);
+}
 
 size_t lf_coo_to_csr_workspace_bytes(int64_t nnz, int64_t num_rows, int64_t num_cols) {
     if (nnz <= 0 || num_rows <= 0 || num_cols <= 0) return 256;

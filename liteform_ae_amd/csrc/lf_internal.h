@@ -20,6 +20,17 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 }  // namespace lf
 
+#ifdef __HIPCC__
+#include <hip/hip_runtime.h>
+namespace lf {
+// Structural check of caller-supplied CSR (or BSR block) index arrays on the GPU, behind
+// lf_csr_check and in front of lf_csr_spmm / lf_bsr_spmm; `what` names the arrays in the
+// error message.  Synchronises `s`.
+int csr_check(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values, int64_t num_rows,
+              int64_t num_cols, int64_t nnz, void* d_scratch, int32_t* h_flags, const char* what, hipStream_t s);
+}  // namespace lf
+#endif
+
 #define LF_REQUIRE(cond, status, ...)                  \
     do {                                               \
         if (!(cond)) return lf::fail(status, __VA_ARGS__); \

@@ -252,19 +252,37 @@ extern "C" int lf_search_bucket_config(const int64_t* h_stats, const int64_t* h_
 //   C        rows * n * 4 bytes written by partition 0, 8 bytes per feature and touched row
 //            (read-modify-write) by every later partition,
 //   slabs    8 bytes per slot and per ELL row.
-// Everything crosses the fabric, which moves kFabricBytesPerPs at best; the part that has to
-// come from HBM as scattered rows moves at kHbmBytesPerPs.  A share h of the gathers is served
-// by the 256 MB memory-side cache: h = kMallShare * 256 MB / (bytes of B one pass touches),
-// at most 1, less the first touches (1 / uses per row of B).  The launch takes the longer of
-// the two, times a penalty when a window reads 256 bytes or less out of a wider row (the
-// partial rows use the fabric worse: x (1 + beta * log2(row bytes / g)^2)), plus a fixed cost.
-// Fitted on 150 measured shapes; the fastest predicted shape is within 3 % of the fastest
-// measured one on every matrix and feature size of the fit.
+// The part of B that one launch can touch is slice = (columns of the partition) * g bytes.
+// Three levels serve the gathers:
+//   * each XCD's 4 MB L2 holds a share h2 = kL2Share * 4 MB / slice of the slice (at most 1),
+//     less the first touches, which every one of the eight L2s has to make itself
+//     (8 / uses per row of B); hits never leave the XCD, and the L2s deliver kL2BytesPerPs;
+//   * what misses crosses the fabric, which moves kFabricBytesPerPs at best;
+//   * the 256 MB memory-side cache serves a share h = kMallShare * 256 MB / slice of that (at
+//     most 1, less the first touches); the rest comes from HBM as scattered rows at
+//     kHbmBytesPerPs.
+// The launch takes the longest of the three, plus kRowPs per ELL row, times a penalty when a
+// window reads 256 bytes or less out of a wider row (partial rows use HBM worse:
+// x (1 + beta * log2(row bytes / g)^2), scaled by the share that no cache serves), plus a
+// fixed cost: kLaunchMs for the first launch of a product, kNextLaunchMs for every further one
+// (its ramp overlaps the tail of the launch before it).
+//
+// kFabricBytesPerPs .. kNotLastPartition were fitted on 150 measured shapes of matrices whose
+// rows hold 4 - 33 entries on average (1 - 4 partitions); the L2 terms, kRowPs and the split
+// launch cost on 198 shapes of three graphs with 28 - 490 entries per row and 1 - 32
+// partitions, for which the model without an L2 level picked one partition and lost 40 - 80 %
+// against the fastest measured shape (tests/golden/launch_shape_measurements.json holds both
+// sets, and a third one that was measured after the fit and is only predicted).
 constexpr double kHbmBytesPerPs = 5.528;
 constexpr double kMallShare = 0.5534;
 constexpr double kMallBytes = 256.0 * 1048576.0;
+constexpr double kL2BytesPerPs = 20.0;
+constexpr double kL2Share = 1.1;
+constexpr double kL2Bytes = 4.0 * 1048576.0;
+constexpr double kXcdCount = 8.0;
+constexpr double kRowPs = 10.0;
 constexpr double kBeta256 = 0.02, kBeta128 = 0.04, kSmallGather = 1.053;
-constexpr double kLaunchMs = 0.029;
+constexpr double kLaunchMs = 0.029, kNextLaunchMs = 0.006;
 // A partition whose rows of C a later one adds to cannot stream its stores past the caches, and
 // what it leaves there takes room from B (fitted: with it the model's pick is within 2.1 % of the
 // fastest measured shape in every group, without it 3.3 % off for the 2.45M-row graph at N = 256).
@@ -298,13 +316,20 @@ extern "C" int lf_model_spmm_ms(const int64_t* h_stats, int32_t num_parts, int32
         }
         const double slice = cols_p * g;
         const double first = std::min(1.0, cols_p / std::max(nnz, 1.0));
+        const double first_l2 = std::min(1.0, kXcdCount * cols_p / std::max(nnz, 1.0));
         const double h = std::min(1.0, kMallShare * kMallBytes / slice) * (1.0 - first);
+        const double h2 = std::min(1.0, kL2Share * kL2Bytes / slice) * (1.0 - first_l2);
+        const double cached = std::max(h, h2);
+        const double pen = 1.0 + (penalty - 1.0) * (1.0 - cached);
         const double gather = nnz * g;
         const double other = (p == 0 ? (double)num_rows * n * 4.0 : touched * n * 8.0) + slots * 8.0 + ell * 8.0;
-        const double fabric_ps = (gather + other) * penalty / kFabricBytesPerPs;
-        const double hbm_ps = ((1.0 - h) * gather + other) * penalty / kHbmBytesPerPs;
-        ms += std::max(fabric_ps, hbm_ps) * 1e-9 * (p + 1 < num_parts ? kNotLastPartition : 1.0) + kLaunchMs;
+        const double l2_ps = (gather + other) / kL2BytesPerPs;
+        const double fabric_ps = ((1.0 - h2) * gather + other) * pen / kFabricBytesPerPs;
+        const double hbm_ps = ((1.0 - cached) * gather + other) * pen / kHbmBytesPerPs;
+        ms += (std::max(l2_ps, std::max(fabric_ps, hbm_ps)) + ell * kRowPs) * 1e-9 *
+                  (p + 1 < num_parts ? kNotLastPartition : 1.0) +
+              kNextLaunchMs;
     }
-    *h_ms = ms * n_windows;
+    *h_ms = ms * n_windows + (kLaunchMs - kNextLaunchMs);
     return LF_OK;
 }

@@ -1012,7 +1012,10 @@ plan_chunks_kernel(const int32_t* __restrict__ rows, const int32_t* __restrict__
         } else {
             seg = (int)((uint32_t)m >> kMetaLenBits);
             split = seg > 1;
-            if (((long long)seg << log_w) > kCoopSlots) {
+            // The counting pass is enqueued together with the slab checks, before their verdict
+            // has been read: a head that announces more ELL rows than the bucket holds (which the
+            // checks flag and the plan is then refused) must not be followed past the array.
+            if (((long long)seg << log_w) > kCoopSlots && e + seg <= n_rows) {
                 total = ((long long)(seg - 1) << log_w) + (meta[e + seg - 1] & kMetaLenMask);
                 dense = total >= dense_min_slots;
                 if (dense) cs = kDenseChunkSlots;
@@ -1832,9 +1835,9 @@ int lf_spmm_set_windows(lf_spmm_plan* plan, int32_t n_windows) {
     return LF_OK;
 }
 
-int lf_csr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values,
-                int64_t num_rows, int64_t num_cols, int32_t feat_size, int32_t b_dtype,
-                const void* d_B, float* d_C, lf_stream_t stream) {
+int lf_csr_spmm_trusted(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values,
+                        int64_t num_rows, int64_t num_cols, int32_t feat_size, int32_t b_dtype,
+                        const void* d_B, float* d_C, lf_stream_t stream) {
     hipStream_t s = (hipStream_t)stream;
     LF_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31) && num_cols >= 1, LF_ERR_INVALID, "bad shape");
     if (num_rows == 0) return LF_OK;
@@ -1855,6 +1858,24 @@ int lf_csr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const float* 
     ks.csr<<<grid, kWG, 0, s>>>(d_indptr, d_indices, d_values, num_rows, a);
     LF_HIP(hipGetLastError());
     return LF_OK;
+}
+
+int lf_csr_spmm(const int32_t* d_indptr, const int32_t* d_indices, const float* d_values,
+                int64_t num_rows, int64_t num_cols, int64_t nnz, int32_t feat_size, int32_t b_dtype,
+                const void* d_B, float* d_C, void* d_scratch, lf_stream_t stream) {
+    // arguments first, so that a bad feature size or operand is reported without touching the GPU
+    LF_REQUIRE(num_rows >= 0 && num_rows < (1ll << 31) && num_cols >= 1, LF_ERR_INVALID, "bad shape");
+    if (num_rows > 0) {
+        LF_REQUIRE(d_indptr && d_B && d_C, LF_ERR_INVALID, "null argument");
+        LF_REQUIRE(b_dtype == LF_DTYPE_F32 || b_dtype == LF_DTYPE_BF16, LF_ERR_INVALID, "unknown B dtype %d", b_dtype);
+        int lpr, ch;
+        if (int rc = feature_shape(feat_size, b_dtype, &lpr, &ch)) return rc;
+    }
+    // no gather before the index arrays have passed
+    if (int rc = lf::csr_check(d_indptr, d_indices, nullptr, num_rows, num_cols, nnz, d_scratch, nullptr, "lf_csr_spmm",
+                               (hipStream_t)stream))
+        return rc;
+    return lf_csr_spmm_trusted(d_indptr, d_indices, d_values, num_rows, num_cols, feat_size, b_dtype, d_B, d_C, stream);
 }
 
 int lf_spmm_time_ms(lf_spmm_plan* plan, const void* d_B, float* d_C, int32_t warmup, int32_t repeat,

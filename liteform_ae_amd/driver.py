@@ -6,9 +6,13 @@ the column-partition count is chosen, the bucket-width search is timed (``time_b
 the hyb format is composed and the fused kernel is timed (``time_exe_our(ms)``).
 
 Differences: the reference predicts the format (CELL or BCSR) and the partition count with
-RandomForest models; the partition model is not distributed and the BSR path is outside
-this library, so every matrix is run as CELL and the partition count is measured
-(``choose_num_partitions``) or given.  Extra columns report GFLOP/s and compose time.
+RandomForest models, of which the partition model is not distributed.  Here the format is
+CELL unless ``select_format`` says otherwise (the BSR and CSR branches of the reference's
+driver, proc05.spmm.end-to-end.py:191-261, run through ``bench_bsrmm`` / ``bench_naive``), and
+the partition count comes, together with the number of feature windows, from the launch-shape
+model (``predict_launch_shape``), or is given.  ``num_parts_override`` stands where the
+reference's driver overrides its predictor by matrix name (proc05.spmm.end-to-end.py:145-148).
+Extra columns report GFLOP/s, feature windows and compose time.
 
     python -m liteform_ae_amd.driver --synthetic cfg2 --feat 32 64 128
     python -m liteform_ae_amd.driver --dataset path/to/matrix.mtx
@@ -26,6 +30,9 @@ import scipy.sparse as sp
 from .format_matrix_market import MTX
 
 FEAT_SIZES = (32, 64, 128, 256, 512)        # proc05.spmm.end-to-end.py:141
+# the partition counts the reference's driver sets by hand, whatever its predictor says
+# (proc05.spmm.end-to-end.py:145-148)
+REFERENCE_NUM_PARTS_OVERRIDE = {"ppi": 16, "proteins": 32}
 
 
 def _run_block_or_csr(g, fa, feat, fmt_name):
@@ -54,10 +61,14 @@ def _run_block_or_csr(g, fa, feat, fmt_name):
 
 
 def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="reference",
-                   check_correctness=False, out_csv=None, keep_values=False, select_format=None):
+                   check_correctness=False, out_csv=None, keep_values=False, select_format=None,
+                   num_parts_override=None):
     """Runs the flow for an iterable of MTX objects and returns a pandas DataFrame with the
     reference's columns.  ``num_parts``: None = from the launch-shape model per (matrix, feature size); an int;
-    or a callable ``(g, feat_size) -> int``.  ``select_format``: None = CELL for every
+    or a callable ``(g, feat_size) -> int``.  ``num_parts_override``: a mapping from matrix name
+    to a partition count that replaces whatever ``num_parts`` gave for that matrix, as the
+    reference's driver does for two of its graphs (``REFERENCE_NUM_PARTS_OVERRIDE``; such a
+    matrix runs in one feature window).  ``select_format``: None = CELL for every
     matrix; or a callable ``g -> "CELL" | "BSR" | "CSR"`` standing in for the reference's
     format-selection model (proc05.spmm.end-to-end.py:133)."""
     import pandas as pd
@@ -94,6 +105,8 @@ def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="
                 parts, windows = int(num_parts(g, feat)), 1
             else:
                 parts, windows = int(num_parts), 1
+            if num_parts_override and g.name in num_parts_override:    # proc05:145-148
+                parts, windows = int(num_parts_override[g.name]), 1
             time_parts = time.perf_counter() - t0
             print(f"name: {g.name} num_parts: {parts} feature_windows: {windows} time(s): {time_parts}")
 
@@ -113,7 +126,7 @@ def run_end_to_end(matrices, feat_sizes=FEAT_SIZES, num_parts=None, cost_model="
                     y_ndarray = g.dot(x.numpy())
                 else:
                     indptr, indices, _ = g.adj_tensors("csr")
-                    ones = sp.csr_matrix((np.ones(len(indices), dtype=np.float32), indices, indptr), shape=g.coo_mtx.shape)
+                    ones = sp.csr_matrix((np.ones(len(indices), dtype=np.float32), indices, indptr), shape=(g.num_src_nodes(), g.num_dst_nodes()))
                     y_ndarray = ones.dot(x.numpy())
             compose_ms = float("nan")
             try:
@@ -157,7 +170,10 @@ def main(argv=None):
     ap.add_argument("--synthetic", nargs="*", default=[], help="synthetic workloads: cfg1 .. cfg5")
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--feat", type=int, nargs="*", default=list(FEAT_SIZES))
-    ap.add_argument("--num-parts", type=int, default=0, help="0 = choose by measurement")
+    ap.add_argument("--num-parts", type=int, default=0,
+                    help="column partitions for every matrix (0 = from the launch-shape model)")
+    ap.add_argument("--reference-overrides", action="store_true",
+                    help="partition counts the reference's driver sets by matrix name (ppi: 16, proteins: 32)")
     ap.add_argument("--cost-model", default="reference", choices=["reference", "gfx950"])
     ap.add_argument("--format", default="CELL", choices=["CELL", "BSR", "CSR"],
                     help="format to run every matrix in (the reference chooses it with a model)")
@@ -169,14 +185,15 @@ def main(argv=None):
         from .synthetic import make_workload
         for name in args.synthetic:
             wl = make_workload(name, args.scale)
-            coo = wl.matrix.coo_mtx                             # the reference's matrices are unweighted
-            mats.append(MTX.from_coo(coo.row, coo.col, coo.shape, name=wl.matrix.name))
+            indptr, indices, _ = wl.matrix.adj_tensors("csr")   # the reference's matrices are unweighted
+            mats.append(MTX.from_csr(indptr, indices, wl.shape, name=wl.matrix.name))
     if not mats:
         ap.print_help(sys.stderr)
         return 2
     run_end_to_end(mats, feat_sizes=args.feat, num_parts=args.num_parts or None, cost_model=args.cost_model,
                    check_correctness=args.check, out_csv=args.csv or None,
-                   select_format=(lambda g: args.format) if args.format != "CELL" else None)
+                   select_format=(lambda g: args.format) if args.format != "CELL" else None,
+                   num_parts_override=REFERENCE_NUM_PARTS_OVERRIDE if args.reference_overrides else None)
     return 0
 
 

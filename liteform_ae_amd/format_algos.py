@@ -68,15 +68,18 @@ def _stream():
 
 
 class _DeviceCSR:
-    """CSR arrays of a matrix on the GPU (int32 indices, float32 values), made from the
-    container's COO triplets by lf_coo_to_csr: sorted columns, duplicates summed - the GPU
-    counterpart of the scipy conversion behind adj_tensors("csr")
-    (format_matrix_market.py:74-76)."""
+    """CSR arrays of a matrix on the GPU (int32 indices, float32 values): sorted columns,
+    duplicates summed - the GPU counterpart of the scipy conversion behind
+    adj_tensors("csr") (format_matrix_market.py:74-76).
+
+    Two ways in.  A container made from CSR arrays (``MTX.from_csr``) is uploaded as it is and
+    checked on the GPU (lf_csr_check): if the arrays are canonical already they are the
+    result - no COO triplets on the host, no sort.  Anything else, and a CSR input that turns
+    out unsorted or with duplicates, goes up as COO triplets and is sorted and merged by
+    lf_coo_to_csr.  ``self.path`` says which one was taken ("csr" or "coo")."""
 
     def __init__(self, g):
         torch = _torch()
-        lib = _lib.load()
-        coo = g.coo_mtx
         self.num_rows = int(g.num_src_nodes())
         self.num_cols = int(g.num_dst_nodes())
         # The reference counts degrees from raw COO triplets (format_algos.py:250, 846); they
@@ -84,6 +87,47 @@ class _DeviceCSR:
         self.coo_nnz = int(g.num_edges())
         if self.coo_nnz >= 2**31:
             raise NotImplementedError("matrices with 2^31 or more stored entries are not supported")
+        self._g = g
+        self._seg_deg = {}
+        self._stats_ws = {}          # num_parts -> statistics workspace holding the row bounds
+        src = getattr(g, "_csr_source", None)
+        if src is not None and self._from_csr(src, bool(getattr(g, "_unit_values", False))):
+            self.path = "csr"
+        else:
+            self._from_coo(g.coo_mtx)
+            self.path = "coo"
+        torch.cuda.current_stream().synchronize()
+
+    def _from_csr(self, csr, unit_values: bool) -> bool:
+        """Uploads the CSR arrays; False (nothing kept) when they are not canonical.  Raises
+        ValueError for arrays that are not a CSR structure at all."""
+        torch = _torch()
+        lib = _lib.load()
+        nnz = int(csr.nnz)
+        indptr = torch.from_numpy(np.ascontiguousarray(csr.indptr, dtype=np.int32)).cuda()
+        indices = torch.from_numpy(np.ascontiguousarray(csr.indices, dtype=np.int32)).cuda()
+        values = None if unit_values else torch.from_numpy(np.ascontiguousarray(csr.data, dtype=np.float32)).cuda()
+        scratch = torch.empty(4, dtype=torch.int32, device="cuda")
+        flags = C.c_int32(0)
+        _lib.check(lib.lf_csr_check(_lib.ptr(indptr), _lib.ptr(indices), _lib.ptr(values), self.num_rows, self.num_cols,
+                                    nnz, _lib.ptr(scratch), C.byref(flags), _stream()))
+        if not flags.value & _lib.LF_CSR_CANONICAL:
+            return False
+        self.indptr, self.indices, self.nnz = indptr, indices, nnz
+        self.all_ones = unit_values or bool(flags.value & _lib.LF_CSR_UNIT_VALUES)
+        self._values = values
+        return True
+
+    @property
+    def values(self):
+        """A's values on the device (ones are made on first use when none were uploaded)."""
+        if self._values is None:
+            self._values = _torch().ones(self.nnz, dtype=_torch().float32, device="cuda")
+        return self._values
+
+    def _from_coo(self, coo):
+        torch = _torch()
+        lib = _lib.load()
         row = torch.from_numpy(np.ascontiguousarray(coo.row, dtype=np.int32)).cuda()
         col = torch.from_numpy(np.ascontiguousarray(coo.col, dtype=np.int32)).cuda()
         data = np.asarray(coo.data)
@@ -101,12 +145,9 @@ class _DeviceCSR:
                                      _lib.ptr(indices), _lib.ptr(values), C.byref(out), _stream()))
         self.nnz = int(out.value)
         self.indices = indices[:self.nnz]
-        self.values = values[:self.nnz]
+        self._values = values[:self.nnz]
         # duplicates of unit entries add up to 2, 3, ...: only a duplicate-free unit matrix is "all ones"
         self.all_ones = ones and self.nnz == self.coo_nnz
-        self._g = g
-        self._seg_deg = {}
-        self._stats_ws = {}          # num_parts -> statistics workspace holding the row bounds
 
     def seg_deg(self, num_parts: int):
         """Per-(partition,row) COO degrees on the device, or None when CSR lengths are the same."""
@@ -125,13 +166,20 @@ class _DeviceCSR:
         return self._seg_deg[num_parts]
 
 
+def _matrix_identity(g):
+    """The object whose replacement means "another matrix": the CSR arrays a container was
+    made from, else its COO matrix."""
+    src = getattr(g, "_csr_source", None)
+    return src if src is not None else g.coo_mtx
+
+
 def _device_csr(g) -> _DeviceCSR:
     cached = getattr(g, "_lf_device_csr", None)
-    if cached is not None and cached[0] is g.coo_mtx:
+    if cached is not None and cached[0] is _matrix_identity(g):
         return cached[1]
     dev = _DeviceCSR(g)
     try:
-        object.__setattr__(g, "_lf_device_csr", (g.coo_mtx, dev))
+        object.__setattr__(g, "_lf_device_csr", (_matrix_identity(g), dev))
     except Exception:
         pass
     return dev
@@ -454,8 +502,9 @@ def spmm_csr(g, B, b_dtype: str = "f32", use_values: bool = True):
     out = torch.empty((dev.num_rows, feat), dtype=torch.float32, device="cuda")
     dt = {"f32": _lib.LF_DTYPE_F32, "bf16": _lib.LF_DTYPE_BF16}[b_dtype]
     vals = dev.values if use_values else None
-    _lib.check(lib.lf_csr_spmm(_lib.ptr(dev.indptr), _lib.ptr(dev.indices), _lib.ptr(vals), dev.num_rows,
-                               dev.num_cols, feat, dt, B.data_ptr(), out.data_ptr(), _stream()))
+    # the device arrays were made by lf_coo_to_csr or have passed lf_csr_check: no second check
+    _lib.check(lib.lf_csr_spmm_trusted(_lib.ptr(dev.indptr), _lib.ptr(dev.indices), _lib.ptr(vals), dev.num_rows,
+                                       dev.num_cols, feat, dt, B.data_ptr(), out.data_ptr(), _stream()))
     return out
 
 
@@ -528,6 +577,7 @@ class _DeviceBSR:
         self.indptr = torch.from_numpy(np.ascontiguousarray(bsr_mat.indptr, dtype=np.int32)).cuda()
         self.indices = torch.from_numpy(np.ascontiguousarray(bsr_mat.indices, dtype=np.int32)).cuda()
         self.data = torch.from_numpy(np.ascontiguousarray(bsr_mat.data, dtype=np.float16).reshape(-1)).cuda()
+        self.checked = False          # the first product checks the block index arrays on the GPU
 
 
 def spmm_bsr(bsr, x, block_size: int = 32):
@@ -540,8 +590,15 @@ def spmm_bsr(bsr, x, block_size: int = 32):
     if x.dtype != torch.float16 or not x.is_cuda or not x.is_contiguous() or x.shape[0] != dev.nb * dev.block_size:
         raise ValueError(f"x must be a contiguous CUDA fp16 tensor with {dev.nb * dev.block_size} rows")
     y = torch.empty((dev.mb * dev.block_size, feat), dtype=torch.float16, device="cuda")
-    _lib.check(lib.lf_bsr_spmm(_lib.ptr(dev.indptr), _lib.ptr(dev.indices), _lib.ptr(dev.data), dev.mb, dev.nb,
-                               dev.block_size, feat, x.data_ptr(), y.data_ptr(), _stream()))
+    if not getattr(dev, "checked", False):
+        scratch = torch.empty(4, dtype=torch.int32, device="cuda")
+        _lib.check(lib.lf_bsr_spmm(_lib.ptr(dev.indptr), _lib.ptr(dev.indices), _lib.ptr(dev.data), dev.mb, dev.nb,
+                                   dev.nnzb, dev.block_size, feat, x.data_ptr(), y.data_ptr(), _lib.ptr(scratch),
+                                   _stream()))
+        dev.checked = True
+    else:
+        _lib.check(lib.lf_bsr_spmm_trusted(_lib.ptr(dev.indptr), _lib.ptr(dev.indices), _lib.ptr(dev.data), dev.mb,
+                                           dev.nb, dev.block_size, feat, x.data_ptr(), y.data_ptr(), _stream()))
     return y
 
 
@@ -676,7 +733,16 @@ def pick_launch_shape(predicted: dict):
     return min((k for k, t in predicted.items() if t <= 1.02 * fastest), key=lambda k: (k[0] * k[1], k[0]))
 
 
-def predict_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Sequence[int] = (1, 2, 3, 4),
+# Partition counts the launch-shape model prices.  The reference's predictor and its driver go up
+# to 32 (proc05.spmm.end-to-end.py:145-148: 16 for ppi, 32 for proteins).
+PARTITION_CANDIDATES = (1, 2, 3, 4, 8, 16, 32)
+# More than four partitions pay only where the part of B that one launch reads fits an L2, and
+# each of the eight L2s has to fetch that part itself: a row of B must be used more than eight
+# times for anything to be left to hit.
+DENSE_USES_PER_B_ROW = 8
+
+
+def predict_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Sequence[int] = PARTITION_CANDIDATES,
                          windows: Sequence[int] = None, return_predictions: bool = False):
     """Column-partition count and feature-window count from a model of the MI355X memory
     system, without composing a format or running a kernel.  Takes the place of the
@@ -687,8 +753,10 @@ def predict_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Se
     pointer each, on the GPU) and the share of columns consecutive rows have in common.  A
     structured matrix (stencil, band) reads B through the L2 whatever the shape: one
     partition, one window.  Otherwise lf_model_spmm_ms prices every candidate and
-    ``pick_launch_shape`` takes the cheapest.  Costs well under a millisecond of GPU time where
-    ``choose_launch_shape`` spends hundreds composing and timing."""
+    ``pick_launch_shape`` takes the cheapest; candidates above four partitions are priced only
+    for matrices that use a row of B more than eight times on average.  Costs a few
+    milliseconds of GPU time at most where ``choose_launch_shape`` spends hundreds composing and
+    timing."""
     if windows is None:
         windows = _window_candidates(feat_size, b_dtype)
     rows, cols = int(g.num_src_nodes()), int(g.num_dst_nodes())
@@ -696,8 +764,15 @@ def predict_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Se
     if row_overlap_device(g) >= ROW_OVERLAP_STRUCTURED:
         best = (min(candidates), _structured_windows(feat_size, b_dtype, windows))
     else:
+        dense = int(g.num_edges()) > DENSE_USES_PER_B_ROW * cols
+        few = [p for p in candidates if p <= 4] or [min(candidates)]
         for p in candidates:
-            stats, _ = bucket_statistics(g, p, with_columns=False)
+            if p not in few and not dense:
+                continue
+            try:
+                stats, _ = bucket_statistics(g, p, with_columns=False)
+            except ValueError:
+                continue
             for w in windows:
                 predicted[(p, w)] = model_spmm_ms(stats, w, rows, cols, feat_size, b_dtype)
         best = pick_launch_shape(predicted)
@@ -731,7 +806,7 @@ def _window_candidates(feat_size: int, b_dtype: str) -> List[int]:
     return [w for w in (1, 2, 4, 8) if feat_size % w == 0 and feat_size // w >= 64 and (feat_size // w) % step == 0] or [1]
 
 
-def choose_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Sequence[int] = (1, 2, 3, 4),
+def choose_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Sequence[int] = PARTITION_CANDIDATES,
                         windows: Sequence[int] = None, cost_model: str = "gfx950", runs: int = 5,
                         return_timings: bool = False):
     """Column-partition count and feature-window count by measurement: composes the format
@@ -766,7 +841,7 @@ def choose_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Seq
     return (best, timings) if return_timings else best
 
 
-def choose_num_partitions(g, feat_size: int, b_dtype: str = "f32", candidates: Sequence[int] = (1, 2, 3, 4),
+def choose_num_partitions(g, feat_size: int, b_dtype: str = "f32", candidates: Sequence[int] = PARTITION_CANDIDATES,
                           cost_model: str = "gfx950", runs: int = 5, return_timings: bool = False):
     """Column-partition count by measurement for a single pass over the features
     (choose_launch_shape with one window)."""

@@ -54,10 +54,12 @@ class MTX:
     """
 
     def __init__(self, filename):
+        self._coo = None
         self._csr = None
+        self._csr_source = None       # the CSR matrix this container was made from (from_csr), as given
+        self._unit_values = False     # from_csr without data: every stored value is 1
         if filename is None:
             self.name = None
-            self.coo_mtx = None
         elif filename in _GRAPH_DATASETS:
             raise RuntimeError(
                 f"dataset '{filename}' is downloaded through dgl/ogb in the reference; "
@@ -69,6 +71,22 @@ class MTX:
             coo = sp.coo_matrix(mmread(filename))
             coo.data = np.ones(len(coo.data))          # format_matrix_market.py:63-64
             self.coo_mtx = coo
+
+    # ``coo_mtx`` is the reference's one data attribute (format_matrix_market.py:44-46).  A
+    # container made from CSR arrays keeps them and builds the COO view only when it is asked
+    # for, so that a CSR input can go to the GPU as it is.
+    @property
+    def coo_mtx(self):
+        if self._coo is None and self._csr_source is not None:
+            self._coo = self._csr_source.tocoo()
+        return self._coo
+
+    @coo_mtx.setter
+    def coo_mtx(self, value):
+        self._coo = value
+        self._csr = None                               # cached views follow the COO
+        self._csr_source = None
+        self._unit_values = False
 
     # ---- constructors without a file -------------------------------------------------
     @classmethod
@@ -84,26 +102,33 @@ class MTX:
 
     @classmethod
     def from_csr(cls, indptr, indices, shape, data=None, name=None):
+        """Container around CSR arrays, kept as they are (no copy for int32 / float32 input).
+        ``data=None`` stores ones, like every matrix of the reference."""
         indptr = np.asarray(indptr)
         indices = np.asarray(indices)
-        if data is None:
-            data = np.ones(len(indices))
-        csr = sp.csr_matrix((np.asarray(data), indices, indptr), shape=shape)
+        unit = data is None
+        if unit:
+            data = np.ones(len(indices), dtype=np.float32)
         m = cls(None)
         m.name = name
-        m.coo_mtx = csr.tocoo()
+        m._csr_source = sp.csr_matrix((np.asarray(data), indices, indptr), shape=shape)
+        m._unit_values = unit
         return m
-
-    def __setattr__(self, key, value):
-        if key == "coo_mtx":
-            object.__setattr__(self, "_csr", None)   # cached CSR follows the COO
-        object.__setattr__(self, key, value)
 
     # ---- the reference's accessors ----------------------------------------------------
     def _csr_view(self):
+        """Canonical CSR (sorted columns, duplicates summed): what coo.tocsr() gives
+        (format_matrix_market.py:74-76)."""
         if self._csr is None:
-            object.__setattr__(self, "_csr", self.coo_mtx.tocsr())
+            src = self._csr_source
+            if src is not None and src.has_canonical_format:
+                self._csr = src
+            else:
+                self._csr = self.coo_mtx.tocsr()
         return self._csr
+
+    def _shape(self):
+        return (self._csr_source if self._coo is None and self._csr_source is not None else self.coo_mtx).shape
 
     def adj_tensors(self, format: str):
         if format == "coo":
@@ -117,12 +142,15 @@ class MTX:
         raise TypeError(f"Format {format} is not suppoted.")
 
     def num_src_nodes(self):
-        return self.coo_mtx.shape[0]
+        return self._shape()[0]
 
     def num_dst_nodes(self):
-        return self.coo_mtx.shape[1]
+        return self._shape()[1]
 
     def num_edges(self):
+        # stored entries: the COO view of a CSR matrix holds exactly its stored entries
+        if self._coo is None and self._csr_source is not None:
+            return self._csr_source.nnz
         return self.coo_mtx.nnz
 
     def dot(self, B):
@@ -148,7 +176,7 @@ class MTX:
     def matrix_features(self):
         """Row-length statistics used by the format selector
         (format_matrix_market.py:153-202)."""
-        num_rows, num_cols = self.coo_mtx.shape
+        num_rows, num_cols = self._shape()
         indptr = self._csr_view().indptr
         per_row = np.diff(indptr)
         avg = np.mean(per_row)
@@ -158,7 +186,7 @@ class MTX:
             "name": self.name,
             "num_rows": num_rows,
             "num_cols": num_cols,
-            "nnz": self.coo_mtx.nnz,
+            "nnz": self.num_edges(),
             "avg_nnz_per_row": avg,
             "min_nnz_per_row": lo,
             "max_nnz_per_row": hi,

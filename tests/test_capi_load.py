@@ -36,7 +36,7 @@ def test_binding_covers_header():
 
 def test_version_and_error_strings():
     lib = _lib.load()
-    assert lib.lf_version() == 100
+    assert lib.lf_version() == 110
     assert lib.lf_status_string(0) == b"ok"
     assert b"single nonzero" in lib.lf_status_string(_lib.LF_ERR_TOO_SMALL)
     # an argument error is reported, not raised as a crash, and leaves a message

@@ -76,7 +76,7 @@ def test_identity_and_empty(fa, torch):
     assert y.shape == (128, 96) and float(y.abs().max()) == 0.0
 
 
-def test_reference_driver_branch(fa, torch):
+def test_reference_driver_branch(fa, torch, monkeypatch):
     """proc05.spmm.end-to-end.py:196-223: pad to a multiple of 32, fp16 BSR, half features."""
     from liteform_ae_amd.format_matrix_market import MTX
     rng = np.random.default_rng(4)
@@ -88,9 +88,8 @@ def test_reference_driver_branch(fa, torch):
     padded = -(-n // 32) * 32
     bsr_weight = g.tobsr_with_padding(shape=(padded, padded), blocksize=(32, 32))
     x = torch.rand(bsr_weight.shape[1], 64).half()
-    import os
-    os.environ["LF_REPEAT"] = "3"
-    os.environ["LF_WARMUP"] = "1"
+    monkeypatch.setenv("LF_REPEAT", "3")
+    monkeypatch.setenv("LF_WARMUP", "1")
     ms = fa.bench_bsrmm(bsr_weight, x, block_size=32)
     assert ms > 0 and np.isfinite(ms)
     y = fa.bench_bsrmm.last_output.cpu().numpy().astype(np.float64)
@@ -100,7 +99,7 @@ def test_reference_driver_branch(fa, torch):
         fa.bench_bsrmm(g.tobsr_with_padding(shape=(1008, 1008), blocksize=(16, 16)), torch.rand(1008, 64).half(), 16)
 
 
-def test_driver_block_and_csr_branches(fa, torch):
+def test_driver_block_and_csr_branches(fa, torch, monkeypatch):
     """proc05.spmm.end-to-end.py:191-261 through the driver: BSR, CSR, and the table's columns."""
     from liteform_ae_amd import driver
     from liteform_ae_amd.format_matrix_market import MTX
@@ -108,9 +107,8 @@ def test_driver_block_and_csr_branches(fa, torch):
     n = 700
     key = np.unique(rng.integers(0, n, size=5000) * n + rng.integers(0, n, size=5000))
     g = MTX.from_coo(key // n, key % n, (n, n), name="toy")
-    import os
-    os.environ["LF_REPEAT"] = "2"
-    os.environ["LF_WARMUP"] = "1"
+    monkeypatch.setenv("LF_REPEAT", "2")
+    monkeypatch.setenv("LF_WARMUP", "1")
     df = driver.run_end_to_end([g], feat_sizes=(32, 64), select_format=lambda m: "BSR")
     assert (df["format"] == "BSR").all() and (df["time_exe_our(ms)"] > 0).all() and (df["num_parts"] == 0).all()
     df = driver.run_end_to_end([g], feat_sizes=(64,), select_format=lambda m: "CSR")

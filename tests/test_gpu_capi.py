@@ -283,6 +283,42 @@ def test_bad_slabs_are_refused_at_plan_creation(env):
     assert create(rows_nd, cols_nd, mask_nd, m)[0] == L.LF_ERR_INVALID
 
 
+def test_a_head_announcing_a_huge_segment_is_refused(env):
+    """A head word that announces 100,000 ELL rows in a 64-wide bucket of a few rows: the
+    announced segment is long enough for the cooperative (chunked) path, whose counting pass
+    is enqueued together with the slab checks; it must not read the meta word of the
+    announced last ELL row, ~400 KB past the array.  Status only."""
+    lib, L, torch = env
+    rng = np.random.default_rng(79)
+    g = skewed_matrix(rng, 300, 5000, mean_deg=4, heavy_rows=2, heavy_len=200, values=False)
+    rows, cols = g.coo_mtx.shape
+    cfg = [[64]]
+    rows_nd, cols_nd, mask_nd = O.build_hyb_format_closed_form(g, cfg)
+    r, c, v = rows_nd[0][0], cols_nd[0][0], mask_nd[0][0]
+    ln = np.maximum(1, (np.asarray(v) != 0).sum(1)).astype(np.int64)
+    meta = np.zeros(len(r), dtype=np.int64)
+    i = 0
+    while i < len(r):
+        j = i
+        while j + 1 < len(r) and r[j + 1] == r[i]:
+            j += 1
+        meta[i] = ln[i] | ((j - i + 1) << 11)
+        for t in range(i + 1, j + 1):
+            meta[t] = ln[t] | ((t - i) << 11) | (1 << 31)
+        i = j + 1
+    for at, announced in ((0, 100_000), (len(r) - 1, (1 << 20) - 1), (len(r) // 2, 70)):
+        m = meta.copy()
+        m[at] = int(m[at] & 0x7FF) | (announced << 11)
+        descs, keep = _tuple_descs(L, torch, [r], [c], [v], cfg[0], [m.astype(np.uint32).view(np.int32)])
+        plan = C.c_void_p()
+        rc = lib.lf_spmm_create(C.byref(plan), descs, 1, 1, rows, cols, 64, 0, None)
+        assert rc == L.LF_ERR_INVALID and "meta" in L.last_error() and not plan.value
+    descs, keep = _tuple_descs(L, torch, [r], [c], [v], cfg[0], [meta.astype(np.uint32).view(np.int32)])
+    plan = C.c_void_p()
+    assert lib.lf_spmm_create(C.byref(plan), descs, 1, 1, rows, cols, 64, 0, None) == 0
+    assert lib.lf_spmm_destroy(plan) == 0
+
+
 def test_derived_meta_of_long_segments(env):
     """Slabs without meta whose widest bucket holds rows split over hundreds of ELL rows (runs
     of equal row ids crossing several 256-row blocks of the derivation pass)."""
@@ -302,3 +338,110 @@ def test_derived_meta_of_long_segments(env):
     ref = O.spmm_csr_f64(indptr, indices, data, (rows, cols), B)
     bound = O.spmm_abs_bound(indptr, indices, data, (rows, cols), B)
     assert (np.abs(out - ref) <= 1e-5 * bound).all()
+
+
+def test_csr_and_bsr_index_arrays_are_checked_before_any_gather(env):
+    """lf_csr_spmm and lf_bsr_spmm take index arrays straight from the caller: an index outside
+    the dense operand, or a row pointer that is not one, must come back as LF_ERR_INVALID with
+    the output untouched - no product kernel may run on such arrays.  Status and output only."""
+    lib, L, torch = env
+    rng = np.random.default_rng(81)
+    rows, cols, feat = 300, 200, 64
+    deg = rng.integers(0, 9, size=rows)
+    indptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int32)
+    nnz = int(indptr[-1])
+    indices = np.concatenate([np.sort(rng.choice(cols, size=d, replace=False)) for d in deg]).astype(np.int32)
+    vals = rng.uniform(-1, 1, size=nnz).astype(np.float32)
+    B = rng.uniform(-1, 1, size=(cols, feat)).astype(np.float32)
+    dB, dV = dev(torch, B, np.float32), dev(torch, vals, np.float32)
+    scratch = torch.zeros(4, dtype=torch.int32, device="cuda")
+    flags = C.c_int32(-1)
+
+    def check(ptr_, idx_, n=nnz, v=None):
+        p, i = dev(torch, ptr_, np.int32), dev(torch, idx_, np.int32)
+        return lib.lf_csr_check(p.data_ptr(), i.data_ptr(), v, rows, cols, n, scratch.data_ptr(), C.byref(flags), None)
+
+    def product(ptr_, idx_, n=nnz):
+        p, i = dev(torch, ptr_, np.int32), dev(torch, idx_, np.int32)
+        out = torch.full((rows, feat), 7.0, device="cuda")
+        rc = lib.lf_csr_spmm(p.data_ptr(), i.data_ptr(), dV.data_ptr(), rows, cols, n, feat, 0, dB.data_ptr(),
+                             out.data_ptr(), scratch.data_ptr(), None)
+        torch.cuda.synchronize()
+        return rc, out
+
+    assert check(indptr, indices, v=dV.data_ptr()) == 0 and flags.value == L.LF_CSR_CANONICAL
+    ones = torch.ones(nnz, device="cuda")
+    assert check(indptr, indices, v=ones.data_ptr()) == 0 and flags.value == L.LF_CSR_CANONICAL | L.LF_CSR_UNIT_VALUES
+    rc, out = product(indptr, indices)
+    assert rc == 0
+    ref = O.spmm_csr_f64(indptr, indices, vals, (rows, cols), B)
+    bound = O.spmm_abs_bound(indptr, indices, vals, (rows, cols), B)
+    assert (np.abs(out.cpu().numpy() - ref) <= 1e-5 * bound).all()
+    # the trusted entry gives the same bits
+    p, i = dev(torch, indptr, np.int32), dev(torch, indices, np.int32)
+    out2 = torch.empty_like(out)
+    assert lib.lf_csr_spmm_trusted(p.data_ptr(), i.data_ptr(), dV.data_ptr(), rows, cols, feat, 0, dB.data_ptr(),
+                                   out2.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+
+    # valid but not canonical: a swapped pair inside a row, a repeated column
+    r = int(np.argmax(deg >= 3))
+    swapped = indices.copy()
+    swapped[indptr[r]], swapped[indptr[r] + 1] = indices[indptr[r] + 1], indices[indptr[r]]
+    assert check(indptr, swapped) == 0 and flags.value == 0
+    repeated = indices.copy()
+    repeated[indptr[r] + 1] = repeated[indptr[r]]
+    assert check(indptr, repeated) == 0 and flags.value == 0
+    assert product(indptr, swapped)[0] == 0                    # still a product one can compute
+
+    bad_cases = []
+    for bad_col in (cols, -1, 2**31 - 1):
+        idx = indices.copy(); idx[nnz // 2] = bad_col
+        bad_cases.append((indptr, idx, nnz))
+    ptr = indptr.copy(); ptr[rows // 2] = ptr[rows // 2 + 1] + 3          # decreasing
+    bad_cases.append((ptr, indices, nnz))
+    ptr = indptr.copy(); ptr[0] = 1                                         # does not start at 0
+    bad_cases.append((ptr, indices, nnz))
+    ptr = indptr.copy(); ptr[-1] = nnz + 1000                               # runs past the arrays
+    bad_cases.append((ptr, indices, nnz))
+    bad_cases.append((indptr, indices, nnz - 1))                            # nnz does not match
+    ptr = indptr.copy(); ptr[3] = -4
+    bad_cases.append((ptr, indices, nnz))
+    for ptr_, idx_, n in bad_cases:
+        assert check(ptr_, idx_, n) == L.LF_ERR_INVALID
+        rc, out = product(ptr_, idx_, n)
+        assert rc == L.LF_ERR_INVALID and "lf_csr_spmm" in L.last_error()
+        assert float(out.min()) == 7.0 and float(out.max()) == 7.0          # nothing was written
+    # no scratch, no check: refused rather than run unchecked
+    p, i = dev(torch, indptr, np.int32), dev(torch, indices, np.int32)
+    out = torch.empty((rows, feat), device="cuda")
+    assert lib.lf_csr_spmm(p.data_ptr(), i.data_ptr(), dV.data_ptr(), rows, cols, nnz, feat, 0, dB.data_ptr(),
+                           out.data_ptr(), None, None) == L.LF_ERR_INVALID
+
+    # BSR: the block structure is a CSR of blocks
+    mb, nb, bs, bfeat = 12, 9, 32, 64
+    bdeg = rng.integers(0, 4, size=mb)
+    bptr = np.concatenate(([0], np.cumsum(bdeg))).astype(np.int32)
+    nnzb = int(bptr[-1])
+    bidx = np.concatenate([np.sort(rng.choice(nb, size=d, replace=False)) for d in bdeg]).astype(np.int32)
+    data = (torch.rand(nnzb * bs * bs, device="cuda") - 0.5).to(torch.float16)
+    X = (torch.rand((nb * bs, bfeat), device="cuda") - 0.5).to(torch.float16)
+
+    def bsr(ptr_, idx_, n=nnzb):
+        p, i = dev(torch, ptr_, np.int32), dev(torch, idx_, np.int32)
+        Y = torch.full((mb * bs, bfeat), 3.0, device="cuda", dtype=torch.float16)
+        rc = lib.lf_bsr_spmm(p.data_ptr(), i.data_ptr(), data.data_ptr(), mb, nb, n, bs, bfeat, X.data_ptr(),
+                             Y.data_ptr(), scratch.data_ptr(), None)
+        torch.cuda.synchronize()
+        return rc, Y
+
+    assert bsr(bptr, bidx)[0] == 0
+    for bad in (nb, -2):
+        idx = bidx.copy(); idx[nnzb // 2] = bad
+        rc, Y = bsr(bptr, idx)
+        assert rc == L.LF_ERR_INVALID and "lf_bsr_spmm" in L.last_error()
+        assert float(Y.float().min()) == 3.0 and float(Y.float().max()) == 3.0
+    ptr = bptr.copy(); ptr[-1] += 5
+    assert bsr(ptr, bidx)[0] == L.LF_ERR_INVALID
+    assert bsr(bptr, bidx, nnzb + 1)[0] == L.LF_ERR_INVALID

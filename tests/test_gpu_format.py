@@ -156,3 +156,71 @@ def test_device_ingest_matches_scipy_tocsr(fa):
     g = MTX.from_coo(np.zeros(0, np.int64), np.zeros(0, np.int64), (7, 9))
     dev = fa._DeviceCSR(g)
     assert dev.nnz == 0 and dev.indptr.cpu().numpy().tolist() == [0] * 8
+
+
+def test_canonical_csr_input_goes_in_as_it_is(fa):
+    """A container made from canonical CSR arrays is uploaded and checked (lf_csr_check), not
+    converted to COO and sorted: same device arrays, statistics and slabs as the COO route."""
+    import scipy.sparse as sp
+    from liteform_ae_amd.format_matrix_market import MTX
+    rng = np.random.default_rng(19)
+    for (nr, nc, deg, weighted) in ((1, 1, 1, False), (700, 900, 9, True), (3000, 40, 5, False), (40, 30000, 200, True)):
+        src = skewed_matrix(rng, nr, nc, mean_deg=deg, heavy_rows=1, values=weighted)
+        indptr, indices, data = src.adj_tensors("csr")
+        g = MTX.from_csr(indptr, indices, (nr, nc), data=data if weighted else None)
+        assert g._coo is None                                   # no COO view was built
+        dev = fa._DeviceCSR(g)
+        assert dev.path == "csr" and g._coo is None
+        ref = fa._DeviceCSR(MTX.from_coo(src.coo_mtx.row, src.coo_mtx.col, (nr, nc), data=data if weighted else None))
+        assert ref.path == "coo"
+        assert dev.nnz == ref.nnz == dev.coo_nnz and dev.all_ones == ref.all_ones == (not weighted)
+        np.testing.assert_array_equal(dev.indptr.cpu().numpy(), ref.indptr.cpu().numpy())
+        np.testing.assert_array_equal(dev.indices.cpu().numpy(), ref.indices.cpu().numpy())
+        np.testing.assert_array_equal(dev.values.cpu().numpy(), ref.values.cpu().numpy())
+        if nr > 1:
+            widths = [[1, 4, 16]] * 2
+            assert_hyb_equal(fa.build_hyb_format(g, widths), O.build_hyb_format_sequential(src, widths))
+            np.testing.assert_array_equal(fa.bucket_statistics(g, 2)[0], stats_from_oracle(src, 2)[0])
+    # float32 ones given as data are recognised on the GPU
+    g = MTX.from_csr(indptr, indices, (nr, nc), data=np.ones(len(indices), dtype=np.float32))
+    assert fa._DeviceCSR(g).all_ones
+    # an empty matrix
+    dev = fa._DeviceCSR(MTX.from_csr(np.zeros(8, np.int32), np.zeros(0, np.int32), (7, 9)))
+    assert dev.path == "csr" and dev.nnz == 0
+
+
+def test_csr_input_that_is_not_canonical_takes_the_sort(fa):
+    """Unsorted columns or duplicates inside a row: the check says so and the arrays go the
+    COO route, ending as scipy's tocsr() has them (format_matrix_market.py:74-76).  Arrays that
+    are no CSR structure at all are refused."""
+    import scipy.sparse as sp
+    from liteform_ae_amd.format_matrix_market import MTX
+    rng = np.random.default_rng(23)
+    nr, nc = 400, 300
+    deg = rng.integers(0, 12, size=nr)
+    indptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int32)
+    for kind in ("unsorted", "duplicates"):
+        if kind == "unsorted":
+            indices = np.concatenate([rng.permutation(nc)[:d] for d in deg]).astype(np.int32)
+        else:
+            indices = np.concatenate([np.sort(rng.integers(0, 6, size=d)) for d in deg]).astype(np.int32)
+        data = rng.uniform(-1, 1, size=len(indices)).astype(np.float32)
+        g = MTX.from_csr(indptr, indices, (nr, nc), data=data)
+        dev = fa._DeviceCSR(g)
+        assert dev.path == "coo"
+        want = sp.csr_matrix((data, indices, indptr), shape=(nr, nc)).tocoo().tocsr()
+        want.sum_duplicates()
+        assert dev.nnz == want.nnz and dev.coo_nnz == len(indices)
+        np.testing.assert_array_equal(dev.indptr.cpu().numpy(), want.indptr)
+        np.testing.assert_array_equal(dev.indices.cpu().numpy(), want.indices)
+        np.testing.assert_allclose(dev.values.cpu().numpy(), want.data, rtol=1e-5, atol=1e-6)
+        widths = [[2, 8]]
+        assert_hyb_equal(fa.build_hyb_format(g, widths), O.build_hyb_format_sequential(g, widths))
+    bad = np.sort(rng.integers(0, nc, size=int(indptr[-1]))).astype(np.int32)
+    bad[5] = nc                                                    # a column outside the matrix
+    m = MTX(None)
+    m._csr_source = sp.csr_matrix((nr, nc), dtype=np.float32)      # placeholder, arrays replaced below
+    m._csr_source.indptr, m._csr_source.indices = indptr, bad
+    m._csr_source.data = np.ones(len(bad), dtype=np.float32)
+    with pytest.raises(ValueError, match="outside"):
+        fa._DeviceCSR(m)

@@ -164,6 +164,7 @@ def test_cfg4_full_size_row_groups(env, monkeypatch):
     B = torch.rand((cols, feat), device="cuda", generator=gen) * 2 - 1
     plan = fa.HybSpMM(fmt, feat)
     assert plan.info["row_group_buckets"] >= 1                           # the stencil takes the shared-gather path
+    assert plan.info["cell_buckets"] >= 1                                # ... as 16-row cells at fp32, N = 256
     C1 = plan.run(B).clone()
     assert torch.equal(C1, plan.run(B))
     plan.close()
@@ -207,8 +208,9 @@ def test_cfg5_full_size_bf16_heavy_rows(env):
     check_statistics(fa, g, 1)
     gen = torch.Generator(device="cuda").manual_seed(5)
     B = (torch.rand((cols, feat), device="cuda", generator=gen) * 2 - 1).to(torch.bfloat16)
-    # the features checked on the host (the whole of B in float64 would be 8 GB)
-    slices = [slice(0, 32), slice(480, 512)]
+    # the features checked on the host (the whole of B in float64 would be 8 GB): both ends and
+    # the seam between the two feature windows
+    slices = [slice(0, 32), slice(240, 272), slice(480, 512)]
     Bh = np.zeros((cols, feat), dtype=np.float32)
     for sl in slices:
         Bh[:, sl] = B[:, sl].to(torch.float32).cpu().numpy()
@@ -223,4 +225,14 @@ def test_cfg5_full_size_bf16_heavy_rows(env):
         assert torch.equal(C1, plan.run(B))
         plan.close()
         check_rows_against_scipy(g, C1, Bh, row_ids, slices)
+        if parts == 1:
+            # the shape the launch-shape model picks for this workload: two feature windows of 256
+            assert fa.predict_launch_shape(g, feat, "bf16") == (1, 2)
+            win = fa.HybSpMM(fmt, feat, "bf16", windows=2)
+            assert win.info["launches"] == 2
+            Cw = win.run(B).clone()
+            assert torch.equal(Cw, win.run(B))
+            win.close()
+            check_rows_against_scipy(g, Cw, Bh, row_ids, slices)
+            del Cw
         del fmt, plan, C1

@@ -264,6 +264,12 @@ def test_partition_chooser_and_driver_table(fa, torch, monkeypatch):
     for keep in (False, True):
         df = driver.run_end_to_end([gw], feat_sizes=(64,), cost_model="gfx950", check_correctness=True, keep_values=keep)
         assert np.isfinite(df["time_exe_our(ms)"]).all(), keep
+    # the reference's driver sets the partition count of two graphs by name, whatever its
+    # predictor says (proc05.spmm.end-to-end.py:145-148): the override table does the same
+    g.name = "ppi"
+    df = driver.run_end_to_end([g, gw], feat_sizes=(64,), check_correctness=True,
+                               num_parts_override=driver.REFERENCE_NUM_PARTS_OVERRIDE)
+    assert df["num_parts"].tolist() == [16, 1] and np.isfinite(df["time_exe_our(ms)"]).all()
 
 
 @pytest.mark.parametrize("feat,b_dtype,windows", [(128, "f32", 2), (256, "f32", 4), (512, "f32", 2), (256, "bf16", 2),
