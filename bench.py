@@ -176,13 +176,14 @@ def compose_cpu_baseline(fa, make_workload, cost_model):
 
 
 def bench_bsr(args):
-    """Block-sparse fp16 side path (bench_bsrmm's kernel): random 32 x 32 block structure."""
-    import scipy.sparse as sp
+    """Block-sparse fp16 side path (bench_bsrmm's kernel): random block structure, blocks of
+    --bsr-block rows and columns, the same number of matrix rows whatever the block size."""
     import torch
     from liteform_ae_amd import format_algos as fa
 
     feat = args.feat or 128
-    mb = nb = max(8, int(round(32768 * args.scale)))
+    bs = args.bsr_block
+    mb = nb = max(8, int(round(32768 * 32 // bs * args.scale)))
     per_row = 8
     rng = np.random.default_rng(1006)
     cols = np.sort(rng.integers(0, nb, size=(mb, per_row)), axis=1)
@@ -193,12 +194,13 @@ def bench_bsr(args):
     indices = cols[keep].astype(np.int32)
     nnzb = len(indices)
     dev = fa._DeviceBSR.__new__(fa._DeviceBSR)
-    dev.block_size, dev.mb, dev.nb, dev.nnzb = 32, mb, nb, nnzb
+    dev.block_size, dev.mb, dev.nb, dev.nnzb = bs, mb, nb, nnzb
     dev.indptr = torch.from_numpy(indptr).cuda()
     dev.indices = torch.from_numpy(indices).cuda()
-    dev.data = (torch.rand(nnzb * 1024, device="cuda") - 0.5).to(torch.float16)
-    x = (torch.rand((nb * 32, feat), device="cuda") - 0.5).to(torch.float16)
-    for _ in range(args.warmup):
+    dev.data = (torch.rand(nnzb * bs * bs, device="cuda") - 0.5).to(torch.float16)
+    dev.checked = False                       # the first product checks the index arrays on the GPU
+    x = (torch.rand((nb * bs, feat), device="cuda") - 0.5).to(torch.float16)
+    for _ in range(max(1, args.warmup)):
         fa.spmm_bsr(dev, x)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -215,15 +217,16 @@ def bench_bsr(args):
         b.synchronize()
         ev.append(a.elapsed_time(b))
     kernel_ms = float(np.mean(ev))
-    flops = 2.0 * nnzb * 1024 * feat
-    algo = nnzb * 2048 + nnzb * 4 + (mb + 1) * 4 + nb * 32 * feat * 2 + mb * 32 * feat * 2
-    gath = nnzb * 2048 + nnzb * 4 + (mb + 1) * 4 + nnzb * 32 * feat * 2 + mb * 32 * feat * 2
+    flops = 2.0 * nnzb * bs * bs * feat
+    blk = bs * bs * 2
+    algo = nnzb * blk + nnzb * 4 + (mb + 1) * 4 + nb * bs * feat * 2 + mb * bs * feat * 2
+    gath = nnzb * blk + nnzb * 4 + (mb + 1) * 4 + nnzb * bs * feat * 2 + mb * bs * feat * 2
     print(json.dumps({
-        "metric": "BSR (32x32, fp16) SpMM GFLOP/s", "value": round(flops / (ms * 1e-3) / 1e9, 1), "unit": "GFLOP/s",
+        "metric": f"BSR ({bs}x{bs}, fp16) SpMM GFLOP/s", "value": round(flops / (ms * 1e-3) / 1e9, 1), "unit": "GFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 in, f32 accumulate",
         "data": "synthetic",
-        "config": {"workload": f"bsr: {mb * 32} x {nb * 32}, {nnzb} dense 32x32 blocks (~{per_row} per block row)",
+        "config": {"workload": f"bsr: {mb * bs} x {nb * bs}, {nnzb} dense {bs}x{bs} blocks (~{per_row} per block row)",
                    "feat_size": feat},
         "roofline": {"bound": "hbm", "achieved": round(algo / (kernel_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(algo / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
@@ -253,6 +256,7 @@ def main():
                     help="cost function of the bucket-width search (the reference's, or the MI355X one)")
     ap.add_argument("--widths", default="", help="bucket widths instead of the searched ones, "
                     "e.g. '1,2,4,8;1,2,4' (partitions separated by ';')")
+    ap.add_argument("--bsr-block", type=int, default=32, choices=[16, 32, 64], help="--workload bsr: block size")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--copy-calibration", action="store_true",

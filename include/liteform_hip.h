@@ -117,7 +117,9 @@ int lf_row_features(const int32_t* d_indptr, int64_t num_rows, void* d_scratch,
  * (device memory, int64 [4], 8-byte aligned) receives {min, max, sum, sum of squares} in stream
  * order.  num_rows above LF_ROW_FEATURES_STATIC_MAX_ROWS is refused with LF_ERR_UNSUPPORTED.
  * All calls on one GPU share that GPU's array: calls that overlap there (two streams, two
- * threads) race and must be serialised by the caller. */
+ * threads) race and must be serialised by the caller.  The first call on a device asks the
+ * runtime for the array's address there (hipGetSymbolAddress): make one call outside any
+ * stream capture before recording the function into a graph. */
 #define LF_ROW_FEATURES_STATIC_MAX_ROWS 2147483646LL
 int lf_row_features_static(const int32_t* d_indptr, int64_t num_rows, int64_t* d_out /* [4] */,
                            lf_stream_t stream);
@@ -324,10 +326,15 @@ int lf_coo_to_csr(const int32_t* d_coo_row, const int32_t* d_coo_col, const floa
                   lf_stream_t stream);
 
 /* Block-sparse SpMM on the matrix cores, the counterpart of bench_bsrmm's kernel
- * (format_algos.py:1182-1643): Y = A_bsr . X with 32 x 32 fp16 blocks (scipy BSR layout:
- * indptr [num_block_rows + 1], indices [nnz blocks], data [nnz blocks][32][32] row-major),
- * X [num_block_cols * 32][feat] fp16, Y [num_block_rows * 32][feat] fp16, fp32 accumulation
- * (the reference accumulates in fp16).  feat_size must be a multiple of 8.
+ * (format_algos.py:1182-1643): Y = A_bsr . X with square fp16 blocks of block_size = 16, 32 or
+ * 64 rows (scipy BSR layout: indptr [num_block_rows + 1], indices [nnz blocks], data
+ * [nnz blocks][block_size][block_size] row-major), X [num_block_cols * block_size][feat] fp16,
+ * Y [num_block_rows * block_size][feat] fp16, fp32 accumulation (the reference accumulates in
+ * fp16).  The reference's schedule takes any multiple of 16 (format_algos.py:1581-1582) and its
+ * driver passes 32 (proc05.spmm.end-to-end.py:205); here the sizes are those whose block rows
+ * fill whole 16- or 32-row matrix-instruction tiles with one tile shape (48, 80, ... would mix
+ * the two): others return LF_ERR_UNSUPPORTED.  feat_size must be a multiple of 8; X, Y and the
+ * block data 16-byte aligned.
  * lf_bsr_spmm checks the block index arrays like lf_csr_check (d_scratch: 16 bytes of device
  * memory; synchronises for the verdict) and returns LF_ERR_INVALID without launching the
  * product when they fail; lf_bsr_spmm_trusted only enqueues the kernel, for arrays that have

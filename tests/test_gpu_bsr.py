@@ -1,4 +1,4 @@
-"""Block-sparse fp16 SpMM (32 x 32 blocks, MFMA) against scipy BSR in float64.
+"""Block-sparse fp16 SpMM (blocks of 16, 32 or 64, MFMA) against scipy BSR in float64.
 
 Tolerance: inputs are exact fp16, products are accumulated in fp32 and the result is rounded
 to fp16 once: |Y - ref| <= 2^-10 |ref| + 1e-5 * sum|a||x| + 1e-7."""
@@ -23,7 +23,7 @@ def torch():
     return torch
 
 
-def random_bsr(rng, mb, nb, blocks_per_row, empty_rows=0, fill=1.0):
+def random_bsr(rng, mb, nb, blocks_per_row, empty_rows=0, fill=1.0, bs=32):
     indptr = [0]
     indices = []
     for i in range(mb):
@@ -32,17 +32,17 @@ def random_bsr(rng, mb, nb, blocks_per_row, empty_rows=0, fill=1.0):
         indices.extend(cols.tolist())
         indptr.append(len(indices))
     # fp16-representable values held as float32 (scipy's sparse containers refuse float16)
-    data = rng.uniform(-1, 1, size=(len(indices), 32, 32)).astype(np.float16).astype(np.float32)
+    data = rng.uniform(-1, 1, size=(len(indices), bs, bs)).astype(np.float16).astype(np.float32)
     if fill < 1.0:
         data[rng.random(data.shape) > fill] = 0
     return sp.bsr_matrix((data, np.array(indices, dtype=np.int32), np.array(indptr, dtype=np.int32)),
-                         shape=(mb * 32, nb * 32))
+                         shape=(mb * bs, nb * bs))
 
 
 def check(fa, torch, a, feat, seed=0):
     rng = np.random.default_rng(seed)
     x = rng.uniform(-1, 1, size=(a.shape[1], feat)).astype(np.float16)
-    y = fa.spmm_bsr(a, torch.from_numpy(x).cuda()).cpu().numpy().astype(np.float64)
+    y = fa.spmm_bsr(a, torch.from_numpy(x).cuda(), block_size=a.blocksize[0]).cpu().numpy().astype(np.float64)
     ref = O.spmm_bsr_f64(a, x)
     bound = O.spmm_bsr_abs_bound(a, x)
     tol = 2.0 ** -10 * np.abs(ref) + 1e-5 * bound + 1e-7
@@ -51,29 +51,36 @@ def check(fa, torch, a, feat, seed=0):
     assert worst <= 0, f"excess {worst}, max err {np.abs(y - ref).max()}"
 
 
+@pytest.mark.parametrize("bs", [16, 32, 64])
 @pytest.mark.parametrize("feat", [8, 32, 64, 128, 200, 256, 512])
-def test_feature_sizes(fa, torch, feat):
-    rng = np.random.default_rng(feat)
-    check(fa, torch, random_bsr(rng, 40, 50, 6, empty_rows=3), feat, seed=feat)
+def test_feature_sizes(fa, torch, feat, bs):
+    rng = np.random.default_rng(feat + bs)
+    check(fa, torch, random_bsr(rng, 40, 50, 6, empty_rows=3, bs=bs), feat, seed=feat)
 
 
-def test_shapes_and_fill(fa, torch):
-    rng = np.random.default_rng(2)
-    check(fa, torch, random_bsr(rng, 1, 1, 1), 128)
-    check(fa, torch, random_bsr(rng, 300, 7, 7), 128)                 # dense block rows
-    check(fa, torch, random_bsr(rng, 7, 300, 40), 64)                 # long block rows
-    check(fa, torch, random_bsr(rng, 100, 100, 5, fill=0.05), 128)    # sparse inside the blocks
+@pytest.mark.parametrize("bs", [16, 32, 64])
+def test_shapes_and_fill(fa, torch, bs):
+    rng = np.random.default_rng(2 + bs)
+    check(fa, torch, random_bsr(rng, 1, 1, 1, bs=bs), 128)
+    check(fa, torch, random_bsr(rng, 300, 7, 7, bs=bs), 128)                 # dense block rows
+    check(fa, torch, random_bsr(rng, 7, 300, 40, bs=bs), 64)                 # long block rows
+    check(fa, torch, random_bsr(rng, 100, 100, 5, fill=0.05, bs=bs), 128)    # sparse inside the blocks
 
 
-def test_identity_and_empty(fa, torch):
+@pytest.mark.parametrize("bs", [16, 32, 64])
+def test_identity_and_empty(fa, torch, bs):
     n = 64 * 32
-    eye = sp.identity(n, dtype=np.float32, format="csr").tobsr(blocksize=(32, 32))
+    eye = sp.identity(n, dtype=np.float32, format="csr").tobsr(blocksize=(bs, bs))
     x = torch.rand((n, 96), device="cuda").to(torch.float16)
-    assert torch.equal(fa.spmm_bsr(eye, x), x)
-    empty = sp.bsr_matrix((np.zeros((0, 32, 32), np.float32), np.zeros(0, np.int32), np.zeros(5, np.int32)),
-                          shape=(4 * 32, 64 * 32))
-    y = fa.spmm_bsr(empty, x)
-    assert y.shape == (128, 96) and float(y.abs().max()) == 0.0
+    assert torch.equal(fa.spmm_bsr(eye, x, block_size=bs), x)
+    empty = sp.bsr_matrix((np.zeros((0, bs, bs), np.float32), np.zeros(0, np.int32), np.zeros(5, np.int32)),
+                          shape=(4 * bs, n))
+    y = fa.spmm_bsr(empty, x, block_size=bs)
+    assert y.shape == (4 * bs, 96) and float(y.abs().max()) == 0.0
+    # a permutation of block columns with one entry per row: every output row is one row of x
+    perm = np.random.default_rng(bs).permutation(n)
+    pm = sp.csr_matrix((np.ones(n, np.float32), (np.arange(n), perm)), shape=(n, n)).tobsr(blocksize=(bs, bs))
+    assert torch.equal(fa.spmm_bsr(pm, x, block_size=bs), x[torch.from_numpy(perm).cuda()])
 
 
 def test_reference_driver_branch(fa, torch, monkeypatch):
@@ -95,8 +102,17 @@ def test_reference_driver_branch(fa, torch, monkeypatch):
     y = fa.bench_bsrmm.last_output.cpu().numpy().astype(np.float64)
     ref = O.spmm_bsr_f64(bsr_weight, x.numpy())
     assert (np.abs(y - ref) <= 2.0 ** -10 * np.abs(ref) + 1e-5 * O.spmm_bsr_abs_bound(bsr_weight, x.numpy()) + 1e-7).all()
+    # the other block sizes the reference's schedule can take (any multiple of 16,
+    # format_algos.py:1581-1582): 16 and 64 are served, the rest is refused
+    for bs, side in ((16, 1008), (64, 1024)):
+        w = g.tobsr_with_padding(shape=(side, side), blocksize=(bs, bs))
+        xb = torch.rand(side, 64).half()
+        assert fa.bench_bsrmm(w, xb, block_size=bs) > 0
+        y = fa.bench_bsrmm.last_output.cpu().numpy().astype(np.float64)
+        ref = O.spmm_bsr_f64(w, xb.numpy())
+        assert (np.abs(y - ref) <= 2.0 ** -10 * np.abs(ref) + 1e-5 * O.spmm_bsr_abs_bound(w, xb.numpy()) + 1e-7).all()
     with pytest.raises(NotImplementedError):
-        fa.bench_bsrmm(g.tobsr_with_padding(shape=(1008, 1008), blocksize=(16, 16)), torch.rand(1008, 64).half(), 16)
+        fa.bench_bsrmm(g.tobsr_with_padding(shape=(1008, 1008), blocksize=(48, 48)), torch.rand(1008, 64).half(), 48)
 
 
 def test_driver_block_and_csr_branches(fa, torch, monkeypatch):

@@ -416,6 +416,26 @@ def test_grid_stencils_are_served_as_cells(fa, torch, feat, windows, b_dtype, mo
     assert info["cell_buckets"] == 0
 
 
+@pytest.mark.parametrize("feat,windows", [(256, 1), (128, 1), (512, 2)])
+def test_cells_in_two_column_partitions(fa, torch, feat, windows, monkeypatch):
+    """Cells in both column partitions: the first partition's cell launch stores C with ordinary
+    stores (the second one reads it again), the second one adds to C and streams its stores.
+    Rows on the grid plane where the partitions meet take terms from both."""
+    rng = np.random.default_rng(300 + feat)
+    for g, widths in ((grid_stencil(rng, (64, 40, 16)), [[32], [32]]),
+                      (grid_stencil(rng, (37, 29, 23)), None),
+                      (grid_stencil(rng, (150, 131)), [[4, 8, 16], [4, 8, 16]])):
+        if widths is None:
+            widths = fa.search_bucket_config(g, 2, fa.CostModelSettings(feat, 2, cost_model="gfx950"))
+        C1, info = check(fa, torch, g, widths, feat, "f32", seed=feat, windows=windows)
+        assert info["cell_buckets"] >= 2, (widths, info)              # at least one bucket of either partition
+        monkeypatch.setenv("LF_ROW_GROUPS", "0")
+        C0, info0 = check(fa, torch, g, widths, feat, "f32", seed=feat, windows=windows)
+        monkeypatch.delenv("LF_ROW_GROUPS")
+        assert info0["row_group_buckets"] == 0
+        assert np.abs(C1 - C0).max() <= 2e-5
+
+
 @pytest.mark.parametrize("feat", [96, 160, 224])
 def test_feature_counts_that_leave_lanes_unused_stay_with_row_groups(fa, torch, feat):
     """160 features take 40 of 64 lanes: the lane layout of the 256-feature kernels, but not the

@@ -55,3 +55,37 @@ def test_static_scratch_rejects_oversize_and_null():
     assert rc == _lib.LF_ERR_UNSUPPORTED and "at most" in _lib.last_error()
     rc = lib.lf_row_features_static(d_indptr.data_ptr(), 1, None, None)
     assert rc == _lib.LF_ERR_INVALID
+
+
+def test_static_scratch_inside_a_hip_graph():
+    """The use the entry point is there for: recorded into a HIP graph (after one eager call on
+    the device, which looks up the array's address) and replayed on changing data, with eager
+    work and synchronisations between the replays; every replay against lf_row_features."""
+    import torch
+    from liteform_ae_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(12)
+    num_rows = 50_000
+    d_indptr = torch.zeros(num_rows + 1, dtype=torch.int32, device="cuda")
+    d_out = torch.zeros(4, dtype=torch.int64, device="cuda")
+    _lib.check(lib.lf_row_features_static(d_indptr.data_ptr(), num_rows, d_out.data_ptr(),
+                                          torch.cuda.current_stream().cuda_stream))         # eager warm-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _lib.check(lib.lf_row_features_static(d_indptr.data_ptr(), num_rows, d_out.data_ptr(),
+                                              torch.cuda.current_stream().cuda_stream))
+    scratch = torch.empty(4, dtype=torch.int64, device="cuda")
+    for hi in (900, 7, 60):
+        deg = rng.integers(0, hi, size=num_rows)
+        indptr = np.concatenate(([0], np.cumsum(deg))).astype(np.int32)
+        d_indptr.copy_(torch.from_numpy(indptr).cuda())
+        d_out.fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = np.zeros(4, dtype=np.int64)
+        _lib.check(lib.lf_row_features(d_indptr.data_ptr(), num_rows, scratch.data_ptr(), want.ctypes.data,
+                                       torch.cuda.current_stream().cuda_stream))
+        np.testing.assert_array_equal(d_out.cpu().numpy(), want)
+        np.testing.assert_array_equal(want, [deg.min(), deg.max(), deg.sum(), (deg.astype(np.int64) ** 2).sum()])
