@@ -206,11 +206,14 @@ int lf_hyb_build(const int32_t* d_indptr, const int32_t* d_indices, const float*
                  lf_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
- * Fused SpMM  C[num_rows][feat] = A_hyb . B[num_cols][feat].  Replaces the kernel that
+ * SpMM  C[num_rows][feat] = A_hyb . B[num_cols][feat].  Replaces the kernel that
  * bench_hyb_with_config builds and launches (format_algos.py:388-605): one launch per
- * column partition walks every bucket of that partition; partitions run in ascending
- * order on the stream, partition 0 stores and later partitions add, so the result does
- * not depend on scheduling and no atomics are used.  C needs no clearing.
+ * column partition (and per feature window, lf_spmm_set_windows) walks every bucket of that
+ * partition - "fused" here means the buckets of a partition, not the partitions; rows served
+ * with shared gathers and the second stage of very long rows have small launches of their
+ * own behind it.  Partitions run in ascending order on the stream, partition 0 stores and
+ * later partitions add, so the result does not depend on scheduling and no atomics are used.
+ * C needs no clearing.
  *
  * A bucket is described the way the reference passes it to the kernel
  * (format_algos.py:552-578: values float32, rows int32, cols int32 row-major), plus the

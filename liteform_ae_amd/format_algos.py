@@ -776,6 +776,11 @@ def predict_launch_shape(g, feat_size: int, b_dtype: str = "f32", candidates: Se
             for w in windows:
                 predicted[(p, w)] = model_spmm_ms(stats, w, rows, cols, feat_size, b_dtype)
         best = pick_launch_shape(predicted)
+        # every statistics pass left its per-partition row bounds behind for the slab builder
+        # ((P + 1) x rows words each); only those of the chosen partition count are of use
+        kept = _device_csr(g)._stats_ws
+        for p in [p for p in kept if p != best[0]]:
+            del kept[p]
     return (best, predicted) if return_predictions else best
 
 
