@@ -111,7 +111,7 @@ __device__ __forceinline__ void ell_tile_narrow(const int2* s_pairs, const int2*
             for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
                 for (int cc = 0; cc < CH; ++cc)
-                    Dense<BT>::load(a.B, (size_t)(uint32_t)c[u] * (size_t)ln.ldb + ln.f[cc], x[u][cc]);
+                    Dense<BT>::load(dense_row<BT>(a.B, ln, cc, c[u]), x[u][cc]);
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
@@ -783,7 +783,7 @@ spmm_rowgroup_kernel(const MergedBucket* __restrict__ buckets, int n_buckets, La
                     float x[U][VEC];
 #pragma unroll
                     for (int u = 0; u < U; ++u)
-                        Dense<BT>::load(a.B, (size_t)(uint32_t)c[u] * (size_t)ln.ldb + ln.f[0], x[u]);
+                        Dense<BT>::load(dense_row<BT>(a.B, ln, 0, c[u]), x[u]);
 #pragma unroll
                     for (int u = 0; u < U; ++u) {
                         const float wr[kGroupRows] = {w[u].x, w[u].y, w[u].z, w[u].w};

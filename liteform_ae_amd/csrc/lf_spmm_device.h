@@ -110,8 +110,9 @@ template <typename BT> struct Dense;
 
 template <> struct Dense<float> {
     static constexpr int kVec = 4;
-    __device__ static __forceinline__ void load(const void* B, size_t elem, float (&x)[4]) {
-        const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(B) + elem);
+    static constexpr int kElemBytes = 4;
+    __device__ static __forceinline__ void load(const char* at, float (&x)[4]) {
+        const float4 v = *reinterpret_cast<const float4*>(at);
         x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
     }
 };
@@ -120,8 +121,9 @@ struct bf16_t { uint16_t bits; };
 
 template <> struct Dense<bf16_t> {
     static constexpr int kVec = 8;
-    __device__ static __forceinline__ void load(const void* B, size_t elem, float (&x)[8]) {
-        const uint4 v = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(B) + elem);
+    static constexpr int kElemBytes = 2;
+    __device__ static __forceinline__ void load(const char* at, float (&x)[8]) {
+        const uint4 v = *reinterpret_cast<const uint4*>(at);
         x[0] = __uint_as_float(v.x << 16); x[1] = __uint_as_float(v.x & 0xFFFF0000u);
         x[2] = __uint_as_float(v.y << 16); x[3] = __uint_as_float(v.y & 0xFFFF0000u);
         x[4] = __uint_as_float(v.z << 16); x[5] = __uint_as_float(v.z & 0xFFFF0000u);
@@ -158,6 +160,18 @@ template <int LPR, int CH, int VEC> struct Lane {
     }
 };
 
+// Where lane `ln` finds its 16 bytes of row `col` of B: the lane's own place in row 0 plus
+// col * (bytes between rows) - one 32 x 32 -> 64-bit multiply-add per gather.  (Indexing in
+// elements, with the row stride as a signed int, cost two 64-bit multiply-adds, two moves and a
+// shift-add per gather: more vector instructions than the four FMAs the gather feeds.)
+template <typename BT, int LPR, int CH>
+__device__ __forceinline__ const char* dense_row(const void* B, const Lane<LPR, CH, Dense<BT>::kVec>& ln, int c,
+                                                 int col) {
+    const char* lane0 = reinterpret_cast<const char*>(B) + (size_t)ln.f[c] * Dense<BT>::kElemBytes;
+    const uint32_t pitch = (uint32_t)ln.ldb * (uint32_t)Dense<BT>::kElemBytes;      // ldb <= 2^20
+    return lane0 + (uint64_t)(uint32_t)col * pitch;
+}
+
 template <int U, int LPR, int CH, typename BT>
 __device__ __forceinline__ void gather_fma(const void* B, const Lane<LPR, CH, Dense<BT>::kVec>& ln,
                                            const int (&col)[U], const float (&val)[U],
@@ -168,7 +182,7 @@ __device__ __forceinline__ void gather_fma(const void* B, const Lane<LPR, CH, De
     for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int c = 0; c < CH; ++c)
-            Dense<BT>::load(B, (size_t)(uint32_t)col[u] * (size_t)ln.ldb + ln.f[c], x[u][c]);
+            Dense<BT>::load(dense_row<BT>(B, ln, c, col[u]), x[u][c]);
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
