@@ -1,5 +1,5 @@
 // Cells: buckets of a structured matrix (stencil, banded, block-structured) rewritten at plan
-// time as groups of up to 16 or 32 rows that lie close together in every direction of the
+// time as groups of up to 16 rows that lie close together in every direction of the
 // underlying grid, with the union of their columns.  Host interface between the plan
 // (lf_spmm.hip) and the cell code (lf_cells.hip).
 #pragma once
@@ -20,6 +20,7 @@ struct LfCellBucket {
     const float4* wq;         // [entries / 4][16] weights: for four consecutive entries and one row of
                               // the cell, the row's values at those columns (0 where it lacks one)
     const int32_t* rows;      // [n_cells * 16] source row of each cell row, -1 where a cell has fewer
+    const uint8_t* euse;      // [entries] bit q: one of the cell's rows 4q .. 4q+3 holds the entry's column
 };
 
 namespace lf {

@@ -8,19 +8,24 @@
 // apart, rows one grid plane apart), with the union of their columns ("merged entries") and,
 // per merged entry, one weight per row of the cell (0 where the row lacks the column).  One
 // 64-lane wavefront owns a cell: it reads each row of B of the union once (16 bytes per lane)
-// and adds weight x row to all 16 accumulator rows at once.  A 4 x 2 x 2 cell of a 27-point
-// stencil reads 96 rows of B for 16 output rows, 6 per row, where row by row it would read 27
-// and four consecutive rows at a time 13.5.
+// and adds weight x row to the accumulator rows that hold the column.  A 2 x 2 x 4 cell of a
+// 27-point stencil reads 96 rows of B for 16 output rows, 6 per row, where row by row it would
+// read 27 and four consecutive rows at a time 13.5.
 //
-// The update "16 rows += 16 weights (x) one row of B" is a rank-1 update, and the matrix
-// pipe has an instruction for exactly that: v_mfma_f32_16x16x1_4b_f32 forms four 16 x 16
-// outer products (fp32 in, fp32 accumulate) per issue.  Written with vector FMAs the same cell
-// takes 18 FMAs and ~30 scalar mask tests per merged entry, and rocprofv3 counters showed the
-// kernel bound by instruction issue (one instruction per ~4.7 cycles and SIMD, 0.88 ms for the
-// 100^3 stencil at N = 256, 0.79 ms with the gathers taken out); with four matrix instructions
-// per entry the arithmetic is no longer what binds.  This is not a GEMM formulation: data
-// layout, gathers and accumulation order are the plain path's, only the accumulate instruction
-// differs, and rows that lack a column add 0 * B (as padded slots do).
+// The update "rows += weights (x) one row of B" is a rank-1 update, and the matrix pipe has
+// instructions for exactly that.  Written with vector FMAs a cell takes 18 FMAs and ~30 scalar
+// mask tests per merged entry, and rocprofv3 counters showed the kernel bound by instruction
+// issue (one instruction per ~4.7 cycles and SIMD, 0.88 ms for the 100^3 stencil at N = 256,
+// 0.79 ms with the gathers taken out).  v_mfma_f32_16x16x1_4b_f32 - four 16 x 16 outer
+// products per issue, all 16 rows at once - brought that to 0.645 ms with the matrix pipe busy
+// 54 % of the time, most of it on zeros: a 27-point stencil fills 432 of a cell's 96 x 16
+// weights.  The kernel now uses v_mfma_f32_4x4x1_16b_f32 - sixteen 4 x 4 outer products per
+// issue, i.e. four rows x 64 lanes, a quarter of the pipe time - once per quarter of the cell
+// (four rows that follow each other) that holds the column, and skips the quarters that do
+// not: 192 of 384 (entry, quarter) pairs for the stencil, 0.63 ms with the same cells, 0.604
+// with cells whose quarters are 2 x 2 x 1.  This is not a GEMM formulation: data layout,
+// gathers and accumulation order are the plain path's, only the accumulate instruction
+// differs, and a row that lacks a column its quarter holds adds 0 * B (as padded slots do).
 //
 // Which rows are neighbours is found from the matrix itself: in a sample of rows, the most
 // frequent differences between two columns of one row are the row distances at which rows
@@ -32,6 +37,7 @@
 #include "lf_cells.h"
 
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 
 #include "lf_spmm_device.h"
@@ -39,6 +45,7 @@
 namespace {
 
 constexpr int kCellRows = 16;              // rows of a cell: the row dimension of the outer-product instruction
+constexpr int kCellQuarters = kCellRows / 4;   // groups of four rows: the row dimension of the 4 x 4 outer-product instruction
 constexpr int kCellBatch = 8;              // merged entries are padded to whole batches of this many
 constexpr int kCellTileCells = 4;          // cells a workgroup is on at a time: one per wavefront (one or two
                                            // per workgroup measured 2 % slower)
@@ -138,6 +145,7 @@ struct CellMergeArgs {
     int32_t* ecol;
     float* wq;                 // float4 per (four consecutive entries, row): [entry / 4][16][entry % 4]
     int32_t* rows_out;         // [n_cells * 16]
+    uint8_t* euse;             // [entries] which quarters of the cell (rows 4q .. 4q+3) hold the entry's column
 };
 
 // Four cells per 64-thread workgroup, one lane per row of a cell.  The rows' slots are staged
@@ -205,6 +213,7 @@ cell_merge_kernel(CellMergeArgs a) {
         const bool any = cmin != 0x7FFFFFFF;       // this group still has columns
         if (__ballot(any) == 0) break;
         const bool mine = any && head == cmin;
+        const unsigned long long holders = __ballot(mine);
         if (write && any) {
             const float v = mine ? s_v[lane * ws + pos] : 0.f;
             pend[0] = (cnt & 3) == 0 ? v : pend[0];
@@ -212,7 +221,12 @@ cell_merge_kernel(CellMergeArgs a) {
             pend[2] = (cnt & 3) == 2 ? v : pend[2];
             pend[3] = (cnt & 3) == 3 ? v : pend[3];
             if ((cnt & 3) == 3) wq4[(size_t)((eo + cnt) >> 2) * G + r] = make_float4(pend[0], pend[1], pend[2], pend[3]);
-            if (r == 0) a.ecol[eo + cnt] = cmin;
+            if (r == 0) {
+                a.ecol[eo + cnt] = cmin;
+                const unsigned h16 = (unsigned)(holders >> (lane & 48)) & 0xFFFFu;
+                a.euse[eo + cnt] = (uint8_t)(((h16 & 0x000Fu) ? 1 : 0) | ((h16 & 0x00F0u) ? 2 : 0) | ((h16 & 0x0F00u) ? 4 : 0) |
+                                             ((h16 & 0xF000u) ? 8 : 0));
+            }
         }
         if (mine) {
             ++pos;
@@ -236,7 +250,10 @@ cell_merge_kernel(CellMergeArgs a) {
     for (int i = cnt; i < m8; ++i) {               // padding entries: the last column again, weight 0
         pend[i & 3] = 0.f;
         if ((i & 3) == 3) wq4[(size_t)((eo + i) >> 2) * G + r] = make_float4(pend[0], pend[1], pend[2], pend[3]);
-        if (r == 0) a.ecol[eo + i] = last_col;
+        if (r == 0) {
+            a.ecol[eo + i] = last_col;
+            a.euse[eo + i] = 0;
+        }
     }
 }
 
@@ -295,6 +312,8 @@ typedef const f32x4 __attribute__((address_space(1)))* GlobalFloat4Ptr;
 typedef const i32x4 __attribute__((address_space(1)))* GlobalInt4Ptr;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef const u32x4 __attribute__((address_space(1)))* GlobalU32x4Ptr;
+typedef const uint32_t __attribute__((address_space(1)))* GlobalU32Ptr;
+typedef const int __attribute__((address_space(1)))* GlobalIntPtr;
 
 // 16 bytes of a row of B as VEC floats
 template <typename BT> __device__ __forceinline__ void unpack_features(const u32x4& r, float (&f)[Dense<BT>::kVec]);
@@ -308,13 +327,26 @@ template <> __device__ __forceinline__ void unpack_features<bf16_t>(const u32x4&
     f[6] = __uint_as_float(r.w << 16); f[7] = __uint_as_float(r.w & 0xFFFF0000u);
 }
 
+// acc[Q] += (weights of rows 4Q .. 4Q+3) (x) (this lane's features), unless no row of the quarter
+// holds the column.  The instruction forms 16 outer products of 4 x 4, one per block of four
+// lanes; with the broadcast field set, every block of a group of 2^CB takes its four weights
+// from block Q of the group - lanes 4Q .. 4Q+3, which hold the weights of rows 4Q .. 4Q+3.
+template <int CB, int Q, int VEC>
+__device__ __forceinline__ void quarter_add(uint32_t quarters, float w, const float (&f)[VEC], f32x4 (&acc)[4][VEC]) {
+    static_assert(kCellQuarters == 4, "one call per quarter");
+    if (__builtin_expect((quarters & (1u << Q)) != 0, 1)) {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) acc[Q][c] = __builtin_amdgcn_mfma_f32_4x4x1f32(w, f[c], acc[Q][c], CB, Q, 0);
+    }
+}
+
 // The SpMM kernel: one workgroup per four cells, one wavefront per cell, XCD-aware like the
 // other kernels (workgroup i runs on XCD i % 8 and takes the i / 8-th tile of that XCD's
 // contiguous share of every bucket).  Per merged entry a wavefront gathers one row of B (lane l
-// holds features VEC*l .. VEC*l+VEC-1) and issues VEC matrix instructions: instruction c takes
-// the entry's 16 weights (lane l supplies the weight of row l % 16) and the c-th feature of
-// every lane, and adds the four 16 x 16 outer products to accumulator c.  In accumulator c,
-// register g of lane l belongs to row 4*(l/16) + g%4 and feature VEC*(16*(g/4) + l%16) + c.
+// holds features VEC*l .. VEC*l+VEC-1) and issues, per quarter that holds the column, VEC
+// matrix instructions: instruction c takes the quarter's four weights and the c-th feature of
+// every lane.  In accumulator [q][c], register i of lane l belongs to row 4q + i and feature
+// VEC*l + c.
 //
 // Columns and weights of a cell are read once and are never in a cache, so every load of them
 // waits out the full memory latency.  Fetched piecemeal next to the gathers they steer (four
@@ -324,26 +356,38 @@ template <> __device__ __forceinline__ void unpack_features<bf16_t>(const u32x4&
 // 4l .. 4l+3; a cell has at most 256) and its weights with up to eight full-width loads that
 // go to LDS; the loop takes columns out of registers (readlane) and weights out of LDS and
 // only ever waits for gathers: 0.67 ms.  Entries are walked in half-batches of four with three
-// in flight (0.645 ms; two 0.67, four 0.65, six 0.66).  C is stored past the caches' retention
-// (non-temporal: 0.765 -> 0.75 ms before the other changes), which leaves more of the L2 to B.
-// Measured on the way: weights straight into LDS with global_load_lds (no staging registers,
-// three wavefronts per SIMD instead of two) 0.75-0.85 ms; three or four wavefronts per SIMD by
-// register limit 0.68 / 0.77 ms.
+// in flight (two 4 % slower, four and five 7 - 8 % slower).  C is stored past the caches'
+// retention (non-temporal: 0.765 -> 0.75 ms before the other changes), which leaves more of
+// the L2 to B.
+// What binds it now (100^3 stencil, N = 256, HIP events): with every gather turned into a cache
+// hit it takes 0.54 ms, without the stores 0.53, with both 0.515 - a wavefront lives ~21 us, of
+// which ~5 pass before its first matrix instruction (offsets, then columns and weights, then the
+// first gathers) and ~3 in the stores, and two wavefronts per SIMD are what the registers allow.
+// Measured against it: weights straight into LDS with global_load_lds (no staging registers,
+// three wavefronts per SIMD) 0.75-0.85 ms; three or four wavefronts per SIMD by register limit
+// 0.68 / 0.77 ms; a grid of resident workgroups that walk every 64th tile and load the next
+// cell's columns and weights behind the last gathers of the current one (loads of a wavefront
+// return in order, so earlier would stall the gathers) 0.70 ms; loads that bring the columns
+// and weights of a tile 8 or 12 ahead into the L2 0.74 ms - every line a wavefront waits for
+// holds a line of the 32 KB L1 for as long as it is under way, and that, not the wavefront's
+// own idle time, is what the loop runs out of.
 constexpr int kCellChunk = 128;            // merged entries whose weights a wavefront holds in LDS at a time
 constexpr int kCellDepth = 3;              // half-batches of gathers in flight
 
 //
 // LPR lanes cover a row of B (64: 256 fp32 or 512 bf16 features per pass; 32 and 16: half and a
 // quarter of that).  With LPR < 64 one gather instruction fetches the rows of E = 64 / LPR
-// consecutive merged entries, one per group of LPR lanes, and the instruction's four blocks
-// fall to different entries: block b belongs to entry b / (4 / E) and feature block b % (4 / E).
-// A lane then holds E partial sums of every output element (entries e, e + E, e + 2E, ...,
-// each in ascending column order), which it adds in the order e = 0 .. E-1 before the store.
-// 27-point stencil on 100^3, cells against four-row groups: fp32 N = 256 0.66 / 1.12 ms,
-// N = 128 0.40 / 0.52 ms, N = 64 0.29 / 0.30 ms (a tie: not worth the rewrite, so 16 lanes per
-// row are not launched); bf16 B doubles the matrix instructions per gathered byte and leaves
-// one wavefront per SIMD (128 accumulator registers): N = 512 / 256 / 128 1.87 / 1.15 / 0.68 ms
-// against 1.51 / 0.72 / 0.41 ms, so bf16 operands stay with the row groups.
+// consecutive merged entries, one per group of LPR lanes, and the instruction's sixteen blocks
+// fall to different entries: the blocks of lanes e * LPR .. (e + 1) * LPR - 1 belong to entry e
+// and take their weights from block q of their own group.  The groups of lanes then hold E
+// partial sums of every output element (entries e, e + E, e + 2E, ..., each in ascending column
+// order), which are added in the order e = 0 .. E-1 before the store.
+// 27-point stencil on 100^3, cells against four-row groups: fp32 N = 256 0.60 / 1.12 ms,
+// N = 128 0.37 / 0.52 ms, N = 64 0.29 / 0.30 ms with the 16 x 16 instruction (a tie: not worth
+// the rewrite, so 16 lanes per row are not launched); bf16 B doubles the matrix instructions per
+// gathered byte and the accumulator registers (one wavefront per SIMD): N = 512 / 256 / 128
+// 1.87 / 1.15 / 0.68 ms against 1.51 / 0.72 / 0.41 ms with the 16 x 16 instruction, so bf16
+// operands stay with the row groups.
 template <typename BT, int LPR>
 __global__ void __launch_bounds__(64 * kCellTileCells)
 spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const void* __restrict__ B,
@@ -353,8 +397,8 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
     constexpr int E = 64 / LPR;                       // merged entries per gather instruction
     constexpr int H = E == 4 ? 2 : 4;                 // gather instructions per half-batch
     constexpr int HE = H * E;                         // merged entries per half-batch: 4 or 8
-    constexpr int NB = 4 / E;                         // feature blocks of 16 lanes per row of B
     constexpr int D = kCellDepth;
+    constexpr int kBroadcast = E == 1 ? 4 : E == 2 ? 3 : 2;   // the weights of one block serve all 16 / 8 / 4 blocks of a group of LPR lanes
     constexpr int kLoads = kCellChunk * 4 / 64;       // full-width loads that bring a chunk's weights
     __shared__ f32x4 s_w[kCellTileCells][kCellChunk * 4];
     const int xcd = blockIdx.x % kXcds;
@@ -367,6 +411,7 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
         // everything that steers the walk is the same for all lanes of a wavefront
         const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
         const int lane = threadIdx.x & 63;
+        const int sub_of_lane = lane / LPR;
         // A wavefront walks kCellsPerWave cells one after the other (at each step the four
         // wavefronts of the workgroup are on four neighbouring cells).  One cell per wavefront
         // measured fastest (100^3 stencil, N = 256: 0.76 / 0.80 / 1.01 ms for 1 / 2 / 4 cells).
@@ -384,13 +429,15 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
         if (m == 0) continue;
         // (pointers read out of the bucket record are generic to the compiler; saying that they
         // are global memory keeps their loads off the LDS counter)
+        const int my_row = reinterpret_cast<GlobalIntPtr>(reinterpret_cast<uintptr_t>(b.rows))[cell * G + (lane & 15)];
         const int cidx = min(4 * lane, m - 4);
         const i32x4 colv = *reinterpret_cast<GlobalInt4Ptr>(reinterpret_cast<uintptr_t>(b.ecol + e0 + cidx));
-        floatx16 acc[VEC];
+        const uint32_t usev = *reinterpret_cast<GlobalU32Ptr>(reinterpret_cast<uintptr_t>(b.euse + e0 + cidx));
+        f32x4 acc[kCellQuarters][VEC];                    // [quarter of the cell][feature of this lane]: rows 4q .. 4q+3
 #pragma unroll
-        for (int c = 0; c < VEC; ++c)
+        for (int q = 0; q < kCellQuarters; ++q)
 #pragma unroll
-            for (int g = 0; g < 16; ++g) acc[c][g] = 0.f;
+            for (int c = 0; c < VEC; ++c) acc[q][c] = f32x4{0.f, 0.f, 0.f, 0.f};
         // A gather is "row base (the same for all lanes, scalar registers) + 16 * lane": no
         // per-load address registers, and the 16 bytes stay packed until they are used.
         const char* b_bytes = reinterpret_cast<const char*>(B);
@@ -407,7 +454,7 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
                 if (i * 64 < mc * 4) wreg[i] = __builtin_nontemporal_load(wsrc + min(i * 64 + lane, mc * 4 - 1));
             const int sub = lane / LPR;                           // which of the E entries of an instruction this lane gathers
             const uint32_t sub_off = (uint32_t)(lane % LPR) * 16u;
-            auto issue = [&](int j, f32x4 (&w)[(HE + 3) / 4], u32x4 (&x)[H], bool with_w) {
+            auto issue = [&](int j, f32x4 (&w)[(HE + 3) / 4], u32x4 (&x)[H], uint32_t (&use)[(HE + 3) / 4], bool with_w) {
                 // (no branch around the loads: the compiler counts outstanding loads per path)
                 const int jj = j < mc ? j : mc - HE;              // past the end: the last half-batch again, unused
                 const int q = (base + jj) >> 2;                   // jj is a multiple of 4: entry n sits in lane n / 4, component n % 4
@@ -418,6 +465,7 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
                     c[t + 1] = __builtin_amdgcn_readlane(colv.y, q + t / 4);
                     c[t + 2] = __builtin_amdgcn_readlane(colv.z, q + t / 4);
                     c[t + 3] = __builtin_amdgcn_readlane(colv.w, q + t / 4);
+                    use[t / 4] = __builtin_amdgcn_readlane(usev, q + t / 4);
                 }
                 if (with_w) {
 #pragma unroll
@@ -437,18 +485,26 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
                     }
                 }
             };
-            auto add_rows = [&](const f32x4 (&w)[(HE + 3) / 4], const u32x4 (&x)[H]) {
+            auto add_rows = [&](const f32x4 (&w)[(HE + 3) / 4], const u32x4 (&x)[H], const uint32_t (&use)[(HE + 3) / 4]) {
 #pragma unroll
                 for (int u = 0; u < H; ++u) {
                     // the weight of this lane's row at the entry this lane's block belongs to
                     float wu = w[(u * E) / 4][(u * E) % 4];
+                    uint32_t quarters = use[(u * E) / 4] >> (8 * ((u * E) % 4));
 #pragma unroll
-                    for (int e = 1; e < E; ++e) wu = sub == e ? w[(u * E + e) / 4][(u * E + e) % 4] : wu;
+                    for (int e = 1; e < E; ++e) {
+                        wu = sub == e ? w[(u * E + e) / 4][(u * E + e) % 4] : wu;
+                        quarters |= use[(u * E + e) / 4] >> (8 * ((u * E + e) % 4));
+                    }
                     float f[VEC];
                     unpack_features<BT>(x[u], f);
-#pragma unroll
-                    for (int c = 0; c < VEC; ++c)
-                        acc[c] = __builtin_amdgcn_mfma_f32_16x16x1f32(wu, f[c], acc[c], 0, 0, 0);
+                    // quarter q: rows 4q .. 4q+3 += their four weights (lanes 4q .. 4q+3 of every
+                    // group of LPR lanes, handed to all blocks of the group) x this lane's features;
+                    // skipped when none of the four rows holds the column (wavefront-uniform test)
+                    quarter_add<kBroadcast, 0, VEC>(quarters, wu, f, acc);
+                    quarter_add<kBroadcast, 1, VEC>(quarters, wu, f, acc);
+                    quarter_add<kBroadcast, 2, VEC>(quarters, wu, f, acc);
+                    quarter_add<kBroadcast, 3, VEC>(quarters, wu, f, acc);
                 }
             };
             // The scheduling fences keep each group of loads ahead of the arithmetic of the
@@ -456,7 +512,8 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
             // their first use and every half-batch waits out the full memory latency.
             f32x4 wr[D][(HE + 3) / 4];
             u32x4 xr[D][H];
-            issue(0, wr[0], xr[0], false);                        // the first gathers leave before the weights are in
+            uint32_t ur[D][(HE + 3) / 4];
+            issue(0, wr[0], xr[0], ur[0], false);                 // the first gathers leave before the weights are in
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < kLoads; ++i)
@@ -467,35 +524,65 @@ spmm_cell_kernel(const LfCellBucket* __restrict__ buckets, int n_buckets, const 
 #pragma unroll
             for (int t = 0; t < (HE + 3) / 4; ++t) wr[0][t] = sw[t * G + (lane & 15)];
 #pragma unroll
-            for (int k = 1; k < D - 1; ++k) issue(k * HE, wr[k], xr[k], true);
+            for (int k = 1; k < D - 1; ++k) issue(k * HE, wr[k], xr[k], ur[k], true);
             for (int j = 0; j < mc; j += D * HE) {
 #pragma unroll
                 for (int k = 0; k < D; ++k) {
-                    issue(j + (D - 1 + k) * HE, wr[(D - 1 + k) % D], xr[(D - 1 + k) % D], true);
+                    issue(j + (D - 1 + k) * HE, wr[(D - 1 + k) % D], xr[(D - 1 + k) % D], ur[(D - 1 + k) % D], true);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (k == 0 || j + k * HE < mc) add_rows(wr[k], xr[k]);
+                    if (k == 0 || j + k * HE < mc) add_rows(wr[k], xr[k], ur[k]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
             __builtin_amdgcn_wave_barrier();
         }
-        // rows of this lane's registers: 4*(lane/16) .. +3
-        const i32x4 my_rows = *reinterpret_cast<GlobalInt4Ptr>(reinterpret_cast<uintptr_t>(b.rows + cell * G + 4 * (lane >> 4)));
-        const int row_of[4] = {my_rows.x, my_rows.y, my_rows.z, my_rows.w};
+        // Register i of acc[q][c] is row 4q + i of the cell at feature VEC * (lane % LPR) + c: a row
+        // leaves as one contiguous run of 16 bytes per lane.
+        if constexpr (E == 1) {
 #pragma unroll
-        for (int g = 0; g < 4 * NB; ++g) {                        // g / 4: feature block, g % 4: row
-            const int row = row_of[g & 3];
-            if (row < 0) continue;
-            float* dst = C + (size_t)row * ldc + VEC * (16 * (g >> 2) + (lane & 15));
+            for (int q = 0; q < kCellQuarters; ++q) {
 #pragma unroll
-            for (int i = 0; i < VEC; i += 4) {
-                f32x4 o = {acc[i][g], acc[i + 1][g], acc[i + 2][g], acc[i + 3][g]};
+                for (int i = 0; i < 4; ++i) {
+                    const int row = __builtin_amdgcn_readlane(my_row, 4 * q + i);
+                    if (row < 0) continue;
+                    float* dst = C + (size_t)row * ldc + VEC * lane;
 #pragma unroll
-                for (int e = 1; e < E; ++e)
-                    o += f32x4{acc[i][g + 4 * NB * e], acc[i + 1][g + 4 * NB * e], acc[i + 2][g + 4 * NB * e],
-                               acc[i + 3][g + 4 * NB * e]};
-                if (accumulate & kAccumulateC) o += *reinterpret_cast<const f32x4*>(dst + i);
-                store_f32x4(dst + i, o, accumulate & kStreamC);
+                    for (int c0 = 0; c0 < VEC; c0 += 4) {
+                        f32x4 o = {acc[q][c0][i], acc[q][c0 + 1][i], acc[q][c0 + 2][i], acc[q][c0 + 3][i]};
+                        if (accumulate & kAccumulateC) o += *reinterpret_cast<const f32x4*>(dst + c0);
+                        store_f32x4(dst + c0, o, accumulate & kStreamC);
+                    }
+                }
+            }
+        } else {
+            // Two entries per gather instruction: lanes 0-31 hold the sums over the even entries,
+            // lanes 32-63 those over the odd ones.  Rows i and i + 2 of a quarter trade halves
+            // (one instruction swaps the upper half of one register with the lower half of
+            // another), after which the lower lanes hold both parts of row i and the upper lanes
+            // both parts of row i + 2; even entries are added first in either.
+            static_assert(E == 2, "the halves of a wavefront are traded");
+#pragma unroll
+            for (int q = 0; q < kCellQuarters; ++q) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const int row_lo = __builtin_amdgcn_readlane(my_row, 4 * q + i);
+                    const int row_hi = __builtin_amdgcn_readlane(my_row, 4 * q + i + 2);
+                    const int row = sub_of_lane ? row_hi : row_lo;
+#pragma unroll
+                    for (int c0 = 0; c0 < VEC; c0 += 4) {
+                        f32x4 o;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            const auto t = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[q][c0 + c][i]),
+                                                                            __float_as_uint(acc[q][c0 + c][i + 2]), false, false);
+                            o[c] = __uint_as_float(t[0]) + __uint_as_float(t[1]);
+                        }
+                        if (row < 0) continue;
+                        float* dst = C + (size_t)row * ldc + VEC * (lane % LPR);
+                        if (accumulate & kAccumulateC) o += *reinterpret_cast<const f32x4*>(dst + c0);
+                        store_f32x4(dst + c0, o, accumulate & kStreamC);
+                    }
+                }
             }
         }
         }
@@ -542,7 +629,18 @@ bool detect_geometry(const std::vector<int32_t>& sample, int n_samples, int n_co
     };
     CellGeom q{};
     q.s1 = 1;
-    const int g3[3] = {4, 2, cell_rows / 8};         // three strides: 4 x 2 x 2
+    // Three strides: 2 x 2 x 4.  Four rows that follow each other in a cell share the matrix
+    // instruction, so the fewer columns such a quarter spans the fewer instructions are spent on
+    // zeros: 2 x 2 x 1 quarters of a 27-point stencil use 48 of the cell's 96 columns, the 4 x 1 x 1
+    // quarters of a 4 x 2 x 2 cell 54 (100^3 stencil, N = 256 / 128: 0.604 / 0.370 ms against
+    // 0.627 / 0.398; 2 x 4 x 2: 0.606 / 0.380; flat cells - 4 x 4 x 1, 8 x 2 x 1 - 0.69 / 0.47).
+    int g3[3] = {2, 2, cell_rows / 4};
+    if (const char* env = getenv("LF_CELL_SHAPE")) {
+        int e0 = 0, e1 = 0, e2 = 0;
+        if (sscanf(env, "%d,%d,%d", &e0, &e1, &e2) == 3 && e0 > 0 && e1 > 0 && e2 > 0 && e0 * e1 * e2 == cell_rows) {
+            g3[0] = e0; g3[1] = e1; g3[2] = e2;
+        }
+    }
     const int g2[2] = {4, cell_rows / 4};            // two strides: 4 x 4
     const long long s2_3 = first_at_least((long long)g3[0]);
     const long long s3_3 = s2_3 ? first_at_least(s2_3 * g3[1]) : 0;
@@ -556,11 +654,13 @@ bool detect_geometry(const std::vector<int32_t>& sample, int n_samples, int n_co
         // cells share come round again a whole layer later, long after they left the L2.  So
         // yb cell rows along y are swept through all z before the next ones, with yb the
         // largest count whose rows of B for one z-step - (yb * g1 + 2) grid lines of s2 / s1
-        // rows in g2 + 2 planes - fit one XCD's 4 MB L2 (100^3 stencil, 1 KB rows: 4; measured
-        // L2 misses 28.4M / 40.8M / 30.7M / 22.2M / 24.4M for plain order / 1 / 2 / 4 / 8).
+        // rows in g2 + 2 planes - fit one XCD's 4 MB L2 (100^3 stencil, 1 KB rows, 4 x 2 x 2
+        // cells: 4; measured L2 misses 28.4M / 40.8M / 30.7M / 22.2M / 24.4M for plain order /
+        // 1 / 2 / 4 / 8).
         const long long line_bytes = (q.s2 / q.s1) * (long long)(q.g2 + 2) * row_bytes;
         const long long lines = line_bytes > 0 ? kL2BytesPerXcd / line_bytes : 0;
         long long yb = (lines - 2) / q.g1;
+        if (lines >= 6) yb = std::max<long long>(yb, 3);          // (measured: 3 or 4 beat 2 where this estimate says 2)
         const char* env_yb = getenv("LF_CELL_YB");
         if (env_yb) yb = atoi(env_yb);
         q.yb = (yb >= 2 && yb < q.n1) ? (int)yb : 0;
@@ -664,6 +764,8 @@ int cells_build(const lf_bucket_desc& b, const int32_t* d_meta, int64_t num_rows
     // ---- offsets and the cells themselves
     int32_t *d_eoff = nullptr, *d_ecol = nullptr, *d_rows_out = nullptr;
     float4* d_wq = nullptr;
+    uint8_t* d_euse = nullptr;
+    if (int rc = cell_alloc(owned, &d_euse, (size_t)rounded)) return rc;
     if (int rc = cell_alloc(owned, &d_eoff, (size_t)n_cells + 1)) return rc;
     if (int rc = cell_alloc(owned, &d_ecol, (size_t)rounded)) return rc;
     if (int rc = cell_alloc(owned, &d_wq, (size_t)rounded / 4 * G)) return rc;
@@ -673,6 +775,7 @@ int cells_build(const lf_bucket_desc& b, const int32_t* d_meta, int64_t num_rows
     ma.ecol = d_ecol;
     ma.wq = reinterpret_cast<float*>(d_wq);
     ma.rows_out = d_rows_out;
+    ma.euse = d_euse;
     cell_merge_kernel<<<(unsigned)lf::ceil_div(n_cells, 4), 64, merge_lds(ma), s>>>(ma);
     LF_HIP(hipGetLastError());
     out->n_cells = n_cells;
@@ -681,6 +784,7 @@ int cells_build(const lf_bucket_desc& b, const int32_t* d_meta, int64_t num_rows
     out->ecol = d_ecol;
     out->wq = d_wq;
     out->rows = d_rows_out;
+    out->euse = d_euse;
     *accepted = true;
     return LF_OK;
 }
