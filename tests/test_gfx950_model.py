@@ -4,7 +4,9 @@ measurements; the fixture tests/golden/launch_shape_measurements.json holds the 
 times, so these tests pin the models' decisions against what the GPU did.  Three sets:
 "cases" (benchmark matrices, 1-4 partitions) and "dense_cases" (three dense-row graphs, 1-32
 partitions) are what the launch-shape constants were fitted to; "validation_cases" (three more
-matrices) were measured after the fit and are only predicted - the out-of-sample error."""
+matrices) were measured after the fit and are only predicted - the out-of-sample error.
+"fold_chains" are what the fold cost's constants were fitted to, "fold_validation" (eight more
+matrices x three feature sizes, tests/golden/measure_fold_chains.py) its out-of-sample check."""
 import json
 import os
 
@@ -55,6 +57,32 @@ def test_model_folds_where_staged_padding_outweighs_the_extra_rows():
 def test_model_keeps_the_initial_width(rows, degree, feat, want):
     cfg, _ = search(uniform_stats(rows, degree), feat)
     assert cfg == [want]
+
+
+def fold_validation_losses():
+    """(key, widths picked, measured ms of the pick, best measured ms of the chain) per held-out chain."""
+    out = []
+    for key, c in MEASURED["fold_validation"].items():
+        stats = np.asarray(c["stats"], dtype=np.int64)[None]
+        cfg = search_from_statistics(stats, None, CostModelSettings(c["feat_size"], 1, cost_model="gfx950"))[0]
+        ms = {tuple(s["widths"]): s["ms"] for s in c["chain"]}
+        assert tuple(cfg) in ms, (key, cfg)              # the pick was timed when the chain was measured
+        out.append((key, cfg, ms[tuple(cfg)], min(ms.values()), max(ms.values())))
+    return out
+
+
+def test_fold_cost_on_matrices_it_was_not_fitted_to():
+    # 24 chains (uniform rows of 9 / 24 / 50 / 70 / 260 entries and three log-normal graphs at
+    # N = 32 / 128 / 512), every state of each chain timed on an MI355X.  The worst state of a
+    # chain is 1.0 - 3.0 times slower than its best; the model's pick loses 1.3 % on average and
+    # 3.9 % at worst (a 0.03 ms product).  Bounds: measured + run-to-run noise.
+    rows = fold_validation_losses()
+    assert len(rows) == 24
+    losses = [picked / best - 1.0 for _, _, picked, best, _ in rows]
+    assert max(losses) <= 0.05, max(zip(losses, (r[0] for r in rows)))
+    assert float(np.mean(losses)) <= 0.02
+    # and the chains are not flat: a careless pick would cost a lot somewhere
+    assert max(worst / best for _, _, _, best, worst in rows) > 2.0
 
 
 def test_model_keeps_power_of_two_widths_on_the_benchmark_graphs():
