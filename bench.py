@@ -51,20 +51,25 @@ KERNEL_SOURCES = ("lf_spmm.hip", "lf_cells.hip", "lf_spmm_device.h")
 
 
 def kernel_source_id():
-    """git blob ids (sha1 of "blob <size>\\0<content>") of the SpMM kernel sources, joined: what a
+    """Identity of the SpMM kernel sources, joined: sha1 of each file with comments and white
+    space taken out (so that rewording a comment does not disown a measurement).  What a
     counter measurement on file has to name to be reported for this build."""
     import hashlib
+    import re
     ids = []
     for name in KERNEL_SOURCES:
-        data = open(os.path.join(ROOT, "liteform_ae_amd", "csrc", name), "rb").read()
-        ids.append(hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest()[:12])
+        text = open(os.path.join(ROOT, "liteform_ae_amd", "csrc", name), "r", encoding="utf-8").read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        text = re.sub(r"//[^\n]*", "", text)
+        text = re.sub(r"\s+", "", text)
+        ids.append(hashlib.sha1(text.encode("utf-8")).hexdigest()[:12])
     return "+".join(ids)
 
 
 def recorded_traffic(workload, feat, parts, windows):
     """L2 <-> fabric bytes per step from the rocprofv3 counter runs summarised in
     profiles/hbm_traffic.md (FETCH_SIZE and WRITE_SIZE, calibrated on a plain copy).  A row
-    counts only if it was taken with the kernel sources of this build (their git blob ids are
+    counts only if it was taken with the kernel sources of this build (their ids are
     in the row); otherwise the figure is unknown and reported as null."""
     key = f"{workload}/N{feat}/P{parts}/W{windows}"
     try:

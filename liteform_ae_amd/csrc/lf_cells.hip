@@ -368,9 +368,10 @@ __device__ __forceinline__ void quarter_add(uint32_t quarters, float w, const fl
 // 0.68 / 0.77 ms; a grid of resident workgroups that walk every 64th tile and load the next
 // cell's columns and weights behind the last gathers of the current one (loads of a wavefront
 // return in order, so earlier would stall the gathers) 0.70 ms; loads that bring the columns
-// and weights of a tile 8 or 12 ahead into the L2 0.74 ms - every line a wavefront waits for
-// holds a line of the 32 KB L1 for as long as it is under way, and that, not the wavefront's
-// own idle time, is what the loop runs out of.  The four wavefronts of a workgroup are on
+// and weights of a tile 8 or 12 ahead into the L2 0.74 ms - an L1 keeps only so many reads
+// under way (70 of 128 bytes on average here, 99 at most on any kernel of this library, by its
+// latency counters; it is stalled on pending data 64 % of its cycles), and that, not the
+// wavefront's own idle time, is what the loop runs out of.  The four wavefronts of a workgroup are on
 // neighbouring cells, and the L1 already serves about a third of their gathers from lines a
 // neighbour asked for (L1 accesses 8.0 GB, its read requests to the L2 4.4 GB); a barrier per
 // turn that keeps the four in step adds 4 % to that and nothing to the time.
