@@ -54,3 +54,33 @@ def test_random_case(seed):
     except ValueError:
         pytest.skip("a column partition holds a single nonzero (the reference raises too)")
     check(fa, torch, g, widths, feat, dt, seed=seed, windows=windows)
+
+
+def random_structured_case(seed):
+    """Stencils and bands in the shapes the 16-row cells take: fp32, 128 or 256 features per pass."""
+    rng = np.random.default_rng(seed)
+    kind = str(rng.choice(["grid3", "grid3", "grid2", "band"]))
+    if kind == "grid3":
+        g = grid_stencil(rng, tuple(int(x) for x in rng.integers(5, 40, size=3)))
+    elif kind == "grid2":
+        g = grid_stencil(rng, tuple(int(x) for x in rng.integers(20, 220, size=2)), reach=int(rng.integers(1, 3)))
+    else:
+        g = banded_matrix(rng, int(rng.integers(4100, 12000)), int(rng.integers(2, 30)), block=int(rng.choice([1, 1, 4])))
+    per, windows = int(rng.choice([128, 256])), int(rng.choice([1, 1, 2]))
+    parts = int(rng.choice([1, 1, 2, 3]))
+    model = str(rng.choice(["gfx950", "reference"]))
+    return g, per * windows, parts, windows, model
+
+
+@pytest.mark.parametrize("seed", range(5000, 5024))
+def test_random_structured_case(seed):
+    # quarters of a cell that lack a column are skipped, cells at the edge of a grid hold fewer than
+    # 16 rows, partitions after the first add to C: all of it varies with the grid's shape
+    import torch
+    from liteform_ae_amd import format_algos as fa
+    g, feat, parts, windows, model = random_structured_case(seed)
+    try:
+        widths = fa.search_bucket_config(g, parts, fa.CostModelSettings(feat, parts, cost_model=model))
+    except ValueError:
+        pytest.skip("a column partition holds a single nonzero (the reference raises too)")
+    check(fa, torch, g, widths, feat, "f32", seed=seed, windows=windows)
