@@ -228,7 +228,7 @@ int lf_hyb_build(const int32_t* d_indptr, const int32_t* d_indices, const float*
  * read of a B row serves several output rows: as groups of four consecutive rows with merged
  * column lists (about 21 bytes per merged entry), or - float32 B, 128 or 256 features per pass - as
  * cells of 16 rows that are neighbours in up to three directions of the underlying grid (the
- * directions are read off the column differences of sampled rows; 68 bytes per merged entry),
+ * directions are read off the column differences of sampled rows; 69 bytes per merged entry),
  * accumulated with the fp32 outer-product matrix instruction.  This costs plan time and memory
  * only where a sample of the bucket shows at least 30 % fewer reads.
  * Rows that hold at least 1/32 of their partition's columns (and 4096 entries), in a partition
