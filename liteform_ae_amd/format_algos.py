@@ -820,7 +820,7 @@ def _structured_windows(feat_size: int, b_dtype: str, windows: Sequence[int]) ->
     """Feature windows for a structured matrix.  Its kernels hold one accumulator per output row
     and feature slice in registers, so they want a row of B to be one 16-byte load per lane:
     256 fp32 features per pass for the 16-row cells (27-point stencil on 100^3, N = 512: one
-    pass 3.29 ms, two passes of 256 1.55 ms), 128 where 256 does not divide N."""
+    pass of four-row groups 3.29 ms, two passes of 256 with cells 1.19 ms), 128 where 256 does not divide N."""
     want = 1
     if b_dtype == "f32":
         if feat_size % 256 == 0:
