@@ -75,7 +75,8 @@ def _upload(array, dtype):
     """A host array as a device tensor of `dtype` (int32 or float32).  Large arrays go through two
     pinned 16 MB staging buffers: the copy into a pinned buffer runs on the host's threads while
     the previous chunk crosses PCIe, which moves a 326 MB index array at 48 GB/s where a plain copy
-    from pageable memory reaches 27."""
+    from pageable memory reaches 27.  The two buffers belong to the process: one upload at a time
+    (the reference's driver is single-threaded too)."""
     global _stage
     torch = _torch()
     src = torch.from_numpy(np.ascontiguousarray(array, dtype=dtype))
